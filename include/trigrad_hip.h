@@ -1,0 +1,142 @@
+/* trigrad_hip.h -- C ABI of libtrigrad_hip.so, the MI355X (gfx950) implementation of
+ * trigrad's differentiable tile rasterizer.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - the library allocates nothing and keeps no state between calls: the
+ *     caller owns every buffer, including workspaces, whose size the
+ *     *_workspace_bytes functions report;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all
+ *     work is enqueued on it and no entry point synchronises;
+ *   - the return value is 0 on success, a negative TG_E_* code for rejected
+ *     arguments, or a positive hipError_t; tg_last_error() describes the last
+ *     failure on the calling thread;
+ *   - data layout is the reference's: vertices (V,4) float32
+ *     (x/w, y/w, z/w, 1/w), indices (M,3) int32, colors (V,3), opacities (V),
+ *     image (H,W,4) with remaining transmittance in channel 3, row 0 at
+ *     y = -1 (reference src/trigrad/wrapper.py:131-141, render.cu:557-562).
+ *
+ * Each entry point names the reference interface it replaces (paths relative
+ * to the reference tree).
+ */
+#ifndef TRIGRAD_HIP_H
+#define TRIGRAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TG_ABI_VERSION 1
+
+#define TG_E_ARG (-1)       /* null pointer, negative size, unsupported tile size */
+#define TG_E_WORKSPACE (-2) /* workspace too small */
+
+/* Status word values written by the kernels that wait on other workgroups. */
+#define TG_STATUS_OK 0u
+#define TG_STATUS_LOOKBACK_TIMEOUT 1u
+
+int tg_version(void);
+const char *tg_last_error(void);
+
+/* Number of tiles of a W x H image (reference render.cu:105-106). */
+int tg_num_tiles(int width, int height, int tile_w, int tile_h);
+
+/* ---- (1) tile binning ------------------------------------------------------- */
+
+/* Per-triangle screen bounds and tile-overlap count: tri_counts[i] = number of
+ * tiles in the clamped tile AABB of triangle i, 0 for a degenerate triangle or
+ * one with a vertex index outside [0, n_vertices).
+ * Replaces count_per_tile / count_per_tile_kernel / touched_tiles
+ * (render.cu:51-76, 90-139); the per-tile histogram of the reference is not
+ * needed by the key pipeline (the tile ranges come out of the sort). */
+int tg_bin_count(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+                 int tile_h, uint32_t *tri_counts, void *stream);
+
+/* Exclusive prefix sum of n uint32 (single pass, decoupled look-back).
+ * out[i] = sum(in[0..i)), *total = sum(in[0..n)).  Replaces the
+ * sum().item() / cumsum_out sequence of per_tile_lists (render.cu:290-295).
+ * `status` (1 uint32, may be NULL) receives TG_STATUS_*; in and out may alias. */
+size_t tg_scan_workspace_bytes(int64_t n);
+int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
+                          size_t workspace_bytes, uint32_t *status, void *stream);
+
+/* Key emission: for triangle i and each tile of its AABB (tile x outer, tile y
+ * inner, render.cu:235-236), at position tri_offsets[i] + local:
+ *   keys[pos]    = (tile_id << 32) | orderable(depth_key)
+ *   payload[pos] = i
+ * where depth_key is the minimum of the triangle's z plane over the triangle
+ * clipped to the tile (1e30 when the clip is empty) and orderable() is the
+ * order-preserving map of float bits to uint32.  Replaces
+ * fill_per_tile_lists_kernel, compute_plane, clip_polygon_to_halfspace
+ * (render.cu:140-270).  n_keys = total of the scan. */
+int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+                int tile_h, const uint32_t *tri_offsets, int64_t n_keys, uint64_t *keys, uint32_t *payload,
+                void *stream);
+
+/* ---- (2) radix sort --------------------------------------------------------- */
+
+/* Stable LSD radix sort of (uint64 key, uint32 value) pairs on key bits
+ * [0, end_bit).  Replaces cub::DeviceSegmentedSort::StableSortPairs as called
+ * by sort_depth_ranges (render.cu:272-284): with the tile id in the high word
+ * one global stable sort yields every tile segment sorted by depth with ties
+ * in input order.  Both buffer pairs are used as ping-pong storage;
+ * *result_in_alt (host) is set to 0 when the sorted data ends in
+ * (keys, values), 1 when it ends in (keys_alt, values_alt). */
+size_t tg_sort_workspace_bytes(int64_t n);
+int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
+                          int end_bit, void *workspace, size_t workspace_bytes, uint32_t *status,
+                          int *result_in_alt, void *stream);
+
+/* ---- (3) tile ranges -------------------------------------------------------- */
+
+/* offsets[t] = first position in sorted_keys whose tile id (key >> 32) is >= t,
+ * for t in [0, n_tiles]; offsets[n_tiles] = n_keys.  Produces the offsets
+ * array that per_tile_lists builds by cumsum (render.cu:292-295). */
+int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int32_t *offsets, void *stream);
+
+/* ---- bary matrices ---------------------------------------------------------- */
+
+/* Row-major 3x3 cartesian-to-barycentric matrix per triangle, out is (M,3,3).
+ * Replaces cartesian_to_bary / cartesian_to_bary_kernel (render.cu:310-337,
+ * 697-711), also exported by the reference as _C.cartesian_to_bary. */
+int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, float *out,
+            void *stream);
+
+/* ---- (4) forward blend ------------------------------------------------------ */
+
+/* One workgroup per tile composites the tile's sorted list.  Replaces
+ * render_forward_kernel and its helpers (render.cu:338-453, 540-619).
+ * Outputs: image (H,W,4), depthmap (H,W), final_weights (H,W), ends (H,W) =
+ * number of blended fragments (the reference's `ends`), and last (H,W) = one
+ * past the tile-list position, relative to the tile's start, of the last
+ * blended entry, and last_depth (H,W) = that entry's pixel depth when
+ * per_pixel_sort is on (render.cu:605-606 lastJ / lastDepth).  last and
+ * last_depth may be NULL; the backward pass needs them.
+ * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
+int tg_render_forward(const float *vertices, const int32_t *indices, const float *colors, const float *opacities,
+                      const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
+                      int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
+                      float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
+                      float *last_depth, void *stream);
+
+/* ---- (5) backward ----------------------------------------------------------- */
+
+/* Accumulates into grad_vertices (V,4), grad_colors (V,3), grad_opacities (V),
+ * which the caller zero-initialises.  Replaces render_backward_kernel /
+ * process_backward (render.cu:455-538, 621-695).  Fragments are visited in
+ * exact reverse blend order. */
+int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
+                       const int32_t *indices, const float *colors, const float *opacities,
+                       const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
+                       const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
+                       const float *last_depth, int width, int height, int tile_w, int tile_h, float early_stopping_threshold,
+                       int per_pixel_sort, int max_layers, float *grad_vertices, float *grad_colors,
+                       float *grad_opacities, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIGRAD_HIP_H */

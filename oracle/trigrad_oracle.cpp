@@ -113,13 +113,16 @@ inline int clip_halfspace(const P2<S> *in, int n_in, P2<S> *out, S nx, S ny, S d
         P2<S> p1 = in[i];
         S d1 = nx * p1.x + ny * p1.y - d;
         bool in1 = d1 >= 0;
-        if (in1 != in0) {
+        // The reference's arrays hold 7 vertices, enough for a convex polygon; a
+        // sliver whose in/out pattern alternates by rounding could exceed that
+        // (undefined behaviour there).  Declared here: capacity 8, the rest dropped.
+        if (in1 != in0 && n_out < 8) {
             S t = d0 / (d0 - d1);
             out[n_out].x = p0.x + t * (p1.x - p0.x);
             out[n_out].y = p0.y + t * (p1.y - p0.y);
             n_out++;
         }
-        if (in1) out[n_out++] = p1;
+        if (in1 && n_out < 8) out[n_out++] = p1;
         p0 = p1; d0 = d1; in0 = in1;
     }
     return n_out;

@@ -1,0 +1,192 @@
+"""GPU parity of the forward blend and the backward pass against the CPU oracle.
+
+Bars (the ones the task states): image within 1e-5 absolute; gradients within
+1e-4 relative + 1e-6 absolute.  The forward kernels evaluate the oracle's
+float32 expression tree operation for operation, so the image is in fact
+expected to be bit-identical; the number of differing values is reported and
+bounded.  The oracle accumulates gradients in float64, the GPU sums float32
+terms with atomics in arbitrary order, hence the gradient tolerance.
+
+Everything here calls the C ABI of libtrigrad_hip.so through trigrad_amd.
+"""
+import numpy as np
+import pytest
+
+from helpers import assert_close, to_device
+from test_gpu_stages import SCENES
+
+pytestmark = pytest.mark.gpu
+
+IMAGE_ATOL = 1e-5
+GRAD_RTOL, GRAD_ATOL = 1e-4, 1e-6
+
+MODES = {
+    "A_default": dict(per_pixel_sort=True, max_layers=32),
+    "A_unlimited": dict(per_pixel_sort=True, max_layers=-1),
+    "A_5_layers": dict(per_pixel_sort=True, max_layers=5),
+    "A_40_layers": dict(per_pixel_sort=True, max_layers=40),
+    "B_unlimited": dict(per_pixel_sort=False, max_layers=-1),
+    "B_3_layers": dict(per_pixel_sort=False, max_layers=3),
+}
+
+
+def _nan_equal(a, b):
+    return np.array_equal(a, b, equal_nan=True)
+
+
+def _forward_both(scene, tw, th, mode, cuda, oracle, thr=1 / 256):
+    from trigrad_amd import _C
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    M = scene["indices"].shape[0]
+    ml = mode["max_layers"] if mode["max_layers"] > 0 else M + 1
+    want = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H, tw, th, thr,
+                         mode["per_pixel_sort"], ml)
+    got = _C.render_forward(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, thr, True,
+                            mode["per_pixel_sort"], ml)
+    return d, want, got, ml
+
+
+def _check_forward(name, want, got):
+    image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status) = got
+    assert int(status.item()) == 0
+    np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
+    np.testing.assert_array_equal(sorted_ids.cpu().numpy(), want["sorted_ids"])
+    img = image.cpu().numpy()
+    finite = np.isfinite(want["image"])
+    assert _nan_equal(np.isnan(img), np.isnan(want["image"])), f"{name}: NaN pattern differs"
+    assert_close(f"{name}: image", np.where(finite, img, 0), np.where(finite, want["image"], 0), 0.0, IMAGE_ATOL)
+    dm = depthmap.cpu().numpy()
+    fin = np.isfinite(want["depthmap"])
+    assert _nan_equal(np.isfinite(dm), fin)
+    assert_close(f"{name}: depthmap", np.where(fin, dm, 0), np.where(fin, want["depthmap"], 0), 1e-5, 1e-5)
+    np.testing.assert_array_equal(ends.cpu().numpy(), want["ends"])
+    np.testing.assert_array_equal(last.cpu().numpy(), want["last"])
+    differing = int((img.view(np.uint32) != want["image"].view(np.uint32)).sum())
+    assert differing == 0, f"{name}: {differing} image values are not bit-identical to the oracle"
+    assert _nan_equal(weights.cpu().numpy(), want["weights"])
+
+
+@pytest.mark.parametrize("mode", sorted(MODES))
+@pytest.mark.parametrize("name", sorted(SCENES))
+def test_forward_matches_oracle(name, mode, cuda, oracle):
+    scene, tw, th = SCENES[name]()
+    _, want, got, _ = _forward_both(scene, tw, th, MODES[mode], cuda, oracle)
+    _check_forward(f"{name}/{mode}", want, got)
+
+
+def _grad_inputs(scene, seed, with_depth):
+    rng = np.random.default_rng(seed)
+    H, W = scene["height"], scene["width"]
+    gi = rng.standard_normal((H, W, 4)).astype(np.float32)
+    gd = rng.standard_normal((H, W)).astype(np.float32) if with_depth else np.zeros((H, W), np.float32)
+    return gi, gd
+
+
+BACKWARD_SCENES = ["config0", "soup_varying_w", "soup_shared", "soup_big_tris", "soup_tile4", "soup_tile32", "soup_tile_8x4",
+                   "squares", "large_triangles", "depth_overlap", "unit_square_negative_z", "grid_mesh", "degenerate"]
+
+
+@pytest.mark.parametrize("with_depth", [False, True])
+@pytest.mark.parametrize("mode", sorted(MODES))
+@pytest.mark.parametrize("name", BACKWARD_SCENES)
+def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
+    import torch
+    from trigrad_amd import _C
+    scene, tw, th = SCENES[name]()
+    m = MODES[mode]
+    d, want, got, ml = _forward_both(scene, tw, th, m, cuda, oracle)
+    W, H = scene["width"], scene["height"]
+    gi, gd = _grad_inputs(scene, 5, with_depth)
+    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                        W, H, tw, th, m["per_pixel_sort"], ml, literal=False)
+    image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
+    out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
+                             d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H, tw, th,
+                             1 / 256, m["per_pixel_sort"], ml, resume=resume)
+    for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
+        g = g.cpu().numpy().astype(np.float64)
+        # float32 summation of n terms: allow rtol on the result plus the rounding
+        # of the largest partial sums (scale of the gradient array)
+        scale = float(np.nanmax(np.abs(w))) if w.size else 0.0
+        assert_close(f"{name}/{mode}: {label}", np.nan_to_num(g), np.nan_to_num(w), GRAD_RTOL, GRAD_ATOL + 2e-6 * scale)
+        assert np.array_equal(np.isnan(g), np.isnan(w))
+    assert float(out[0][:, 2].abs().max()) == 0.0  # z never receives a gradient (render.cu:531-533)
+
+
+def test_default_mode_literal_and_policy_agree(oracle):
+    """With per_pixel_sort on and at most 32 blended fragments the literal
+    reference traversal and the reverse-order policy are the same computation."""
+    from trigrad_amd import scenes as S
+    scene = S.random_soup(300, 64, 64, seed=9, sigma_px=14.0, varying_w=True)
+    W = H = 64
+    fwd = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H)
+    gi, gd = _grad_inputs(scene, 1, True)
+    a = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], fwd, W, H, literal=True)
+    b = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], fwd, W, H, literal=False)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+
+
+def test_render_autograd_end_to_end(cuda, oracle):
+    """trigrad_amd.render + loss.backward() on configuration 0 (both modes)."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import scenes as S
+    scene = S.config(0)
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    for kw in (dict(), dict(per_pixel_sort=False, max_layers=-1)):
+        v = d["vertices"].clone().requires_grad_()
+        c = d["colors"].clone().requires_grad_()
+        o = d["opacities"].clone().requires_grad_()
+        image, depthmap = trigrad_amd.render(v, d["indices"], c, o, W, H, **kw)
+        loss = ((image - d["target"]) ** 2).sum()
+        loss.backward()
+        pps = kw.get("per_pixel_sort", True)
+        ml = kw.get("max_layers", 32)
+        fwd = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H, per_pixel_sort=pps,
+                            max_layers=ml)
+        assert_close("image", image.detach().cpu().numpy(), fwd["image"], 0.0, IMAGE_ATOL)
+        gi = 2.0 * (fwd["image"] - scene["target"])
+        gV, gC, gO = oracle.render_backward(gi, np.zeros((H, W), np.float32), scene["vertices"], scene["indices"], scene["colors"],
+                                            scene["opacities"], fwd, W, H, per_pixel_sort=pps, max_layers=ml)
+        for label, g, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
+            assert_close(label, g.cpu().numpy(), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * float(np.abs(w).max()))
+
+
+def test_record_timing_and_empty_scene(cuda):
+    import torch
+    import trigrad_amd
+    from trigrad_amd import scenes as S
+    d = to_device(S.config(0), cuda)
+    image, depthmap, timings = trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], 256, 256, record_timing=True)
+    assert set(timings) == {"init", "per_tile_lists", "sorting", "bary_transforms", "rasterization"}
+    assert all(t >= 0 for t in timings.values())
+    v = d["vertices"].clone().requires_grad_()
+    empty = torch.empty((0, 3), dtype=torch.int32, device=cuda)
+    image, depthmap = trigrad_amd.render(v, empty, d["colors"], d["opacities"], 64, 48)
+    assert image.shape == (48, 64, 4) and float(image[..., 3].min()) == 1.0 and float(image[..., :3].abs().max()) == 0.0
+    assert torch.isinf(depthmap).all()
+    image.sum().backward()
+    assert float(v.grad.abs().max()) == 0.0
+    image, depthmap, timings = trigrad_amd.render(v, empty, d["colors"], d["opacities"], 64, 48, record_timing=True)
+    assert timings is None
+
+
+def test_argument_errors(cuda):
+    import torch
+    import trigrad_amd
+    from trigrad_amd import scenes as S
+    d = to_device(S.config(0), cuda)
+    v, i, c, o = d["vertices"], d["indices"], d["colors"], d["opacities"]
+    with pytest.raises(ValueError, match="tile_width \\* tile_height must be <= 1024"):
+        trigrad_amd.render(v, i, c, o, 64, 64, 64, 32)
+    with pytest.raises(TypeError, match="vertices must be on cuda"):
+        trigrad_amd.render(v.cpu(), i, c, o)
+    with pytest.raises(TypeError, match="indices must be of type torch.int32"):
+        trigrad_amd.render(v, i.long(), c, o)
+    with pytest.raises(ValueError, match="colors must be of shape"):
+        trigrad_amd.render(v, i, c[:-1], o)
+    with pytest.raises(TypeError, match="opacities must be of type torch.float32"):
+        trigrad_amd.render(v, i, c, o.double())

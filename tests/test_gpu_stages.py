@@ -1,0 +1,192 @@
+"""GPU parity of the integer stages (binning, scan, key emission, radix sort, tile
+ranges) and of the bary matrices against the CPU oracle: bit-exact.
+
+Everything here calls the C ABI of libtrigrad_hip.so through trigrad_amd._C.
+"""
+import numpy as np
+import pytest
+
+from helpers import to_device, u64
+
+pytestmark = pytest.mark.gpu
+
+
+def _scenes():
+    from trigrad_amd import scenes as S
+    out = {
+        "config0": lambda: (S.config(0, with_target=False), 16, 16),
+        "soup_varying_w": lambda: (S.random_soup(3000, 300, 200, seed=1, sigma_px=9.0, varying_w=True), 16, 16),
+        "soup_shared": lambda: (S.random_soup(2000, 257, 131, seed=2, shared=True), 16, 16),
+        "soup_big_tris": lambda: (S.random_soup(400, 128, 128, seed=3, sigma_px=80.0, varying_w=True), 16, 16),
+        "soup_tile4": lambda: (S.random_soup(500, 50, 50, seed=4, sigma_px=5.0), 4, 4),
+        "soup_tile32": lambda: (S.random_soup(800, 200, 150, seed=5, sigma_px=12.0), 32, 32),
+        "soup_tile_8x4": lambda: (S.random_soup(800, 100, 90, seed=6, sigma_px=7.0), 8, 4),
+        "soup_tile_12x20": lambda: (S.random_soup(800, 130, 170, seed=7, sigma_px=7.0), 12, 20),
+        "squares": lambda: (S.overlapping_squares(10), 4, 4),
+        "large_triangles": lambda: (S.large_triangles(3, r=4), 4, 4),
+        "depth_overlap": lambda: (S.depth_overlap(), 16, 16),
+        "unit_square_negative_z": lambda: (S.unit_square(), 16, 16),
+        "overlap_mesh_inf_w": lambda: (S.overlap_mesh(), 16, 16),
+        "grid_mesh": lambda: (S.grid_mesh(40, 40, -0.9, 0.9, -0.9, 0.9, width=96, height=96), 16, 16),
+    }
+    return out
+
+
+def _degenerate_scene():
+    """Zero-area, NaN, infinite, huge and far off-screen triangles mixed with ordinary ones."""
+    from trigrad_amd import scenes as S
+    s = S.random_soup(64, 96, 80, seed=11, sigma_px=10.0, varying_w=True)
+    v = s["vertices"].copy()
+    v[0:3, :2] = v[0, :2]                       # zero area
+    v[3:6, 0] = np.float32("nan")               # NaN
+    v[6, 0] = np.float32("inf")                 # infinite
+    v[9:12, :2] *= np.float32(1e20)             # area overflows to inf
+    v[12:15, 0] += np.float32(5.0)              # entirely right of the screen: clamped into the border tiles
+    v[15:18, :2] = np.array([[-1, -1], [1, -1], [0, 1]], np.float32) * np.float32(3)  # covers everything
+    v[18, :2] = (-1.0, -1.0); v[19, :2] = (-0.75, -1.0); v[20, :2] = (-1.0, -0.5)    # on tile boundaries
+    s["vertices"] = v
+    return s, 16, 16
+
+
+SCENES = _scenes()
+SCENES["degenerate"] = _degenerate_scene
+
+
+@pytest.mark.parametrize("name", sorted(SCENES))
+def test_binning_sort_ranges_bit_exact(name, cuda, oracle):
+    from trigrad_amd import _C
+    scene, tw, th = SCENES[name]()
+    W, H = scene["width"], scene["height"]
+    v, idx = scene["vertices"], scene["indices"]
+    d = to_device(scene, cuda)
+    T = _C.num_tiles(W, H, tw, th)
+
+    tri_counts, tile_counts = oracle.bin_count(v, idx, W, H, tw, th)
+    got_counts = _C.bin_count(d["vertices"], d["indices"], W, H, tw, th)
+    np.testing.assert_array_equal(got_counts.cpu().numpy(), tri_counts)
+
+    offs, total, status = _C.scan_exclusive(got_counts)
+    assert int(status.item()) == 0
+    K = int(total.item())
+    assert K == int(tri_counts.sum())
+    np.testing.assert_array_equal(offs.cpu().numpy(), np.cumsum(tri_counts) - tri_counts)
+
+    em = oracle.bin_emit(v, idx, W, H, tw, th)
+    keys, payload = _C.bin_emit(d["vertices"], d["indices"], offs, K, W, H, tw, th)
+    np.testing.assert_array_equal(u64(keys), em["keys64"])
+    np.testing.assert_array_equal(payload.cpu().numpy(), em["tri"])
+
+    want_keys, want_vals = oracle.sort_pairs_u64(em["keys64"], em["tri"])
+    skeys, svals, sstatus = _C.sort_pairs(keys, payload, _C.key_bits(T))
+    assert int(sstatus.item()) == 0
+    np.testing.assert_array_equal(u64(skeys), want_keys)
+    np.testing.assert_array_equal(svals.cpu().numpy(), want_vals)
+
+    offsets = _C.tile_ranges(skeys, T)
+    np.testing.assert_array_equal(offsets.cpu().numpy(), oracle.tile_ranges(want_keys, T))
+
+    # the same observable through the reference-shaped route: per-tile histogram,
+    # cumsum, slot fill in triangle order, stable segmented sort on float keys
+    ref_offsets, ref_ids, _ = oracle.per_tile_lists(v, idx, W, H, tw, th)
+    np.testing.assert_array_equal(offsets.cpu().numpy(), ref_offsets)
+    np.testing.assert_array_equal(svals.cpu().numpy(), ref_ids)
+    np.testing.assert_array_equal(np.diff(ref_offsets), tile_counts)
+
+    got_bary = _C.cartesian_to_bary(d["vertices"], d["indices"]).cpu().numpy()
+    want_bary = oracle.bary(v, idx)
+    np.testing.assert_array_equal(got_bary.view(np.uint32), want_bary.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 2047, 2048, 2049, 100_003, (1 << 20) + 7])
+def test_scan_matches_cumsum(n, cuda):
+    import torch
+    from trigrad_amd import _C
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, 50, size=n).astype(np.int32)
+    x[rng.integers(0, n, size=max(1, n // 10))] = 0
+    t = torch.from_numpy(x).to(cuda)
+    out, total, status = _C.scan_exclusive(t)
+    assert int(status.item()) == 0
+    np.testing.assert_array_equal(out.cpu().numpy(), np.cumsum(x) - x)
+    assert int(total.item()) == int(x.sum())
+    out2, total2, _ = _C.scan_exclusive(t, out=t)  # in place
+    np.testing.assert_array_equal(out2.cpu().numpy(), np.cumsum(x) - x)
+    assert int(total2.item()) == int(x.sum())
+
+
+def test_scan_empty(cuda):
+    import torch
+    from trigrad_amd import _C
+    out, total, status = _C.scan_exclusive(torch.empty((0,), dtype=torch.int32, device=cuda))
+    assert out.numel() == 0 and int(total.item()) == 0 and int(status.item()) == 0
+
+
+@pytest.mark.parametrize("n,end_bit,distinct", [
+    (1, 64, None), (2, 64, None), (100, 64, None), (4095, 64, None), (4096, 64, None), (4097, 64, None),
+    (100_000, 64, None), (100_000, 45, None), (50_000, 64, 7), (300_000, 40, 1000), ((1 << 20) + 13, 45, None),
+])
+def test_sort_pairs_stable(n, end_bit, distinct, cuda, oracle):
+    """Random keys, optionally drawn from few distinct values so that stability
+    (equal keys keep input order) decides the result; numpy's stable argsort is
+    the library statement of the expected permutation."""
+    import torch
+    from trigrad_amd import _C
+    rng = np.random.default_rng(n + end_bit)
+    if distinct:
+        pool = rng.integers(0, 1 << min(end_bit, 63), size=distinct, dtype=np.uint64)
+        keys = pool[rng.integers(0, distinct, size=n)]
+    else:
+        keys = rng.integers(0, 1 << min(end_bit, 63), size=n, dtype=np.uint64)
+        if end_bit == 64:
+            keys |= rng.integers(0, 2, size=n, dtype=np.uint64) << np.uint64(63)
+    vals = np.arange(n, dtype=np.int32)
+    order = np.argsort(keys, kind="stable")
+    k = torch.from_numpy(keys.view(np.int64).copy()).to(cuda)
+    v = torch.from_numpy(vals.copy()).to(cuda)
+    sk, sv, status = _C.sort_pairs(k, v, end_bit)
+    assert int(status.item()) == 0
+    np.testing.assert_array_equal(u64(sk), keys[order])
+    np.testing.assert_array_equal(sv.cpu().numpy(), vals[order])
+    if n <= 100_000:
+        ok, ov = oracle.sort_pairs_u64(keys, vals)
+        np.testing.assert_array_equal(ok, keys[order])
+        np.testing.assert_array_equal(ov, vals[order])
+
+
+def test_sort_empty_and_zero_bits(cuda):
+    import torch
+    from trigrad_amd import _C
+    k = torch.empty((0,), dtype=torch.int64, device=cuda)
+    v = torch.empty((0,), dtype=torch.int32, device=cuda)
+    sk, sv, status = _C.sort_pairs(k, v, 64)
+    assert sk.numel() == 0 and sv.numel() == 0
+    k = torch.tensor([5, 3, 9], dtype=torch.int64, device=cuda)
+    v = torch.tensor([0, 1, 2], dtype=torch.int32, device=cuda)
+    sk, sv, _ = _C.sort_pairs(k, v, 0)  # no key bits: the identity
+    assert sk.tolist() == [5, 3, 9] and sv.tolist() == [0, 1, 2]
+
+
+def test_tile_ranges_with_empty_tiles(cuda, oracle):
+    import torch
+    from trigrad_amd import _C
+    tiles = np.array([2, 2, 2, 5, 9, 9], dtype=np.uint64)
+    keys = (tiles << np.uint64(32)) | np.arange(6, dtype=np.uint64)
+    t = torch.from_numpy(keys.view(np.int64)).to(cuda)
+    got = _C.tile_ranges(t, 12).cpu().numpy()
+    np.testing.assert_array_equal(got, np.searchsorted(tiles, np.arange(13)))
+    np.testing.assert_array_equal(got, oracle.tile_ranges(keys, 12))
+    empty = _C.tile_ranges(torch.empty((0,), dtype=torch.int64, device=cuda), 7).cpu().numpy()
+    np.testing.assert_array_equal(empty, np.zeros(8, np.int32))
+
+
+def test_out_of_range_indices_are_skipped(cuda):
+    """A triangle naming a vertex outside [0, V) counts no tiles instead of being read."""
+    import torch
+    from trigrad_amd import _C, scenes as S
+    s = S.random_soup(10, 64, 64, seed=3)
+    idx = s["indices"].copy()
+    idx[4, 1] = 10_000
+    idx[7, 0] = -1
+    d = to_device(s, cuda)
+    counts = _C.bin_count(d["vertices"], torch.from_numpy(idx).to(cuda), 64, 64, 16, 16).cpu().numpy()
+    assert counts[4] == 0 and counts[7] == 0 and (np.delete(counts, [4, 7]) > 0).all()

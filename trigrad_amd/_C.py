@@ -1,0 +1,254 @@
+"""Native surface of the renderer: the functions the reference exports from its
+pybind module (src/trigrad/module.cu:8-21, render.h) with the same names and
+argument order, implemented by calling the C ABI of libtrigrad_hip.so on the
+current torch stream.  torch is used for device memory and streams only.
+
+`render_forward` runs the key pipeline the library is built around:
+    bin_count -> scan -> (read K) -> bin_emit -> sort_pairs -> tile_ranges
+    -> cartesian_to_bary -> forward kernel
+and the individual stages are exposed as functions for tests and benchmarks.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+precision = torch.float32  # module.cu:17-21; this build is the float32 one
+
+STAGE_KEYS = ("init", "per_tile_lists", "sorting", "bary_transforms", "rasterization")  # render.cu:723-747
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(t):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise TypeError(f"expected a cuda tensor, got {t.device.type}")
+
+
+def num_tiles(width, height, tile_width, tile_height):
+    return int(_lib.load().tg_num_tiles(width, height, tile_width, tile_height))
+
+
+def key_bits(n_tiles):
+    """Significant bits of a (tile << 32 | depth) key."""
+    return 32 + max(1, int(n_tiles - 1).bit_length())
+
+
+# ---- stages ------------------------------------------------------------------------
+
+def bin_count(vertices, indices, width, height, tile_width, tile_height):
+    """Per-triangle tile-overlap counts, (M,) int32."""
+    _need_cuda(vertices, indices)
+    lib = _lib.load()
+    M = indices.shape[0]
+    counts = torch.empty((M,), dtype=torch.int32, device=vertices.device)
+    with torch.cuda.device(vertices.device):
+        _lib.check(lib.tg_bin_count(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
+                                    _ptr(counts), _stream(vertices)), "tg_bin_count")
+    return counts
+
+
+def scan_exclusive(counts, out=None):
+    """Exclusive prefix sum of an int32 tensor -> (offsets, total (1,) int32, status (1,) int32)."""
+    _need_cuda(counts)
+    lib = _lib.load()
+    n = counts.numel()
+    dev = counts.device
+    out = torch.empty_like(counts) if out is None else out
+    total = torch.empty((1,), dtype=torch.int32, device=dev)
+    status = torch.empty((1,), dtype=torch.int32, device=dev)
+    ws_bytes = int(lib.tg_scan_workspace_bytes(n))
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.tg_scan_exclusive_u32(_ptr(counts), _ptr(out), n, _ptr(total), _ptr(ws), ws_bytes, _ptr(status),
+                                             _stream(counts)), "tg_scan_exclusive_u32")
+    return out, total, status
+
+
+def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, tile_height):
+    """-> (keys (K,) int64 holding uint64 bit patterns, payload (K,) int32) in emission order."""
+    _need_cuda(vertices, indices, tri_offsets)
+    lib = _lib.load()
+    dev = vertices.device
+    keys = torch.empty((n_keys,), dtype=torch.int64, device=dev)
+    payload = torch.empty((n_keys,), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.tg_bin_emit(_ptr(vertices), vertices.shape[0], _ptr(indices), indices.shape[0], width, height, tile_width,
+                                   tile_height, _ptr(tri_offsets), n_keys, _ptr(keys), _ptr(payload), _stream(vertices)),
+                   "tg_bin_emit")
+    return keys, payload
+
+
+def sort_pairs(keys, values, end_bit=64):
+    """Stable sort of (uint64 key, 32-bit value) pairs on key bits [0, end_bit).
+
+    The inputs are used as scratch (their contents are undefined afterwards).
+    -> (sorted_keys, sorted_values, status (1,) int32)
+    """
+    _need_cuda(keys, values)
+    lib = _lib.load()
+    n = keys.numel()
+    dev = keys.device
+    keys_alt = torch.empty_like(keys)
+    values_alt = torch.empty_like(values)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    ws_bytes = int(lib.tg_sort_workspace_bytes(n))
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    in_alt = C.c_int(0)
+    with torch.cuda.device(dev):
+        _lib.check(lib.tg_sort_pairs_u64_u32(_ptr(keys), _ptr(values), _ptr(keys_alt), _ptr(values_alt), n, end_bit, _ptr(ws),
+                                             ws_bytes, _ptr(status), C.byref(in_alt), _stream(keys)), "tg_sort_pairs_u64_u32")
+    if in_alt.value:
+        return keys_alt, values_alt, status
+    return keys, values, status
+
+
+def tile_ranges(sorted_keys, n_tiles):
+    """offsets (T+1,) int32 of the tile segments of a sorted key array."""
+    _need_cuda(sorted_keys)
+    lib = _lib.load()
+    offsets = torch.empty((n_tiles + 1,), dtype=torch.int32, device=sorted_keys.device)
+    with torch.cuda.device(sorted_keys.device):
+        _lib.check(lib.tg_tile_ranges(_ptr(sorted_keys), sorted_keys.numel(), n_tiles, _ptr(offsets), _stream(sorted_keys)),
+                   "tg_tile_ranges")
+    return offsets
+
+
+def cartesian_to_bary(vertices, indices):
+    """(M,3,3) cartesian-to-barycentric matrices (reference _C.cartesian_to_bary, render.cu:697-711)."""
+    _need_cuda(vertices, indices)
+    lib = _lib.load()
+    vertices = vertices.contiguous()
+    indices = indices.contiguous()
+    M = indices.shape[0]
+    out = torch.empty((M, 3, 3), dtype=torch.float32, device=vertices.device)
+    with torch.cuda.device(vertices.device):
+        _lib.check(lib.tg_bary(_ptr(vertices), vertices.shape[0], _ptr(indices), M, _ptr(out), _stream(vertices)), "tg_bary")
+    return out
+
+
+def per_tile_lists(vertices, indices, width, height, tile_width, tile_height):
+    """Binning + sort + ranges -> (sorted_ids (K,) int32, offsets (T+1,) int32, sorted_keys (K,) int64).
+
+    Observable of the reference's per_tile_lists + sort_depth_ranges
+    (render.cu:272-308).  Reads K back from the device once, like the
+    reference's sum().item() (render.cu:290).
+    """
+    T = num_tiles(width, height, tile_width, tile_height)
+    counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
+    tri_offsets, total, status = scan_exclusive(counts, out=counts)
+    host = torch.stack([total[0], status[0]]).cpu()  # the one device->host read of the forward pass
+    K, st = int(host[0]), int(host[1])
+    if st != 0:
+        raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
+    keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height)
+    keys, payload, sort_status = sort_pairs(keys, payload, key_bits(T))
+    offsets = tile_ranges(keys, T)
+    return payload, offsets, keys, sort_status
+
+
+class _StageTimer:
+    """Seconds per stage from events on the current stream (render.cu:11-49)."""
+
+    def __init__(self, disable):
+        self.disable = disable
+        self.marks = []
+
+    def start(self, name):
+        if self.disable:
+            return
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.marks.append((name, ev))
+
+    def stop(self):
+        if self.disable:
+            return {}
+        end = torch.cuda.Event(enable_timing=True)
+        end.record()
+        end.synchronize()
+        evs = [e for _, e in self.marks] + [end]
+        return {name: evs[k].elapsed_time(evs[k + 1]) / 1000.0 for k, (name, _) in enumerate(self.marks)}
+
+
+def render_forward(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                   early_stopping_threshold, disable_timing, per_pixel_sort, max_layers):
+    """Reference _C.render_forward (render.cu:713-763).
+
+    -> (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume)
+    `resume` = (last, last_depth, status): what the backward pass needs to start
+    its reverse traversal, plus the sort's status word.
+    """
+    _need_cuda(vertices, indices, colors, opacities)
+    lib = _lib.load()
+    timer = _StageTimer(disable_timing)
+    dev = vertices.device
+    with torch.cuda.device(dev):
+        timer.start("init")
+        vertices = vertices.contiguous()
+        indices = indices.contiguous()
+        colors = colors.contiguous()
+        opacities = opacities.contiguous()
+        image = torch.empty((height, width, 4), dtype=torch.float32, device=dev)
+        depthmap = torch.empty((height, width), dtype=torch.float32, device=dev)
+        final_weights = torch.empty((height, width), dtype=torch.float32, device=dev)
+        ends = torch.empty((height, width), dtype=torch.int32, device=dev)
+        last = torch.empty((height, width), dtype=torch.int32, device=dev)
+        last_depth = torch.empty((height, width), dtype=torch.float32, device=dev) if per_pixel_sort else None
+
+        timer.start("per_tile_lists")
+        T = num_tiles(width, height, tile_width, tile_height)
+        counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
+        tri_offsets, total, status = scan_exclusive(counts, out=counts)
+        host = torch.stack([total[0], status[0]]).cpu()
+        K, st = int(host[0]), int(host[1])
+        if st != 0:
+            raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
+        keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height)
+
+        timer.start("sorting")
+        keys, sorted_ids, sort_status = sort_pairs(keys, payload, key_bits(T))
+        offsets = tile_ranges(keys, T)
+
+        timer.start("bary_transforms")
+        bary_transforms = cartesian_to_bary(vertices, indices)
+
+        timer.start("rasterization")
+        _lib.check(lib.tg_render_forward(
+            _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
+            width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
+            _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _stream(vertices)),
+            "tg_render_forward")
+        timings = timer.stop()
+    return image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, (last, last_depth, sort_status)
+
+
+def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
+                    image, depthmap, final_weights, ends, width, height, tile_width, tile_height, early_stopping_threshold,
+                    per_pixel_sort, max_layers, resume=None):
+    """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities)."""
+    if resume is None:
+        raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
+    last, last_depth, sort_status = resume
+    _need_cuda(grad_output, vertices)
+    lib = _lib.load()
+    dev = vertices.device
+    with torch.cuda.device(dev):
+        tensors = [t.contiguous() for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
+                                            bary_transforms, image, depthmap, final_weights, ends, last)]
+        grad_vertices = torch.zeros_like(tensors[2])
+        grad_colors = torch.zeros_like(tensors[4])
+        grad_opacities = torch.zeros_like(tensors[5])
+        _lib.check(lib.tg_render_backward(
+            *[_ptr(t) for t in tensors], _ptr(last_depth), width, height, tile_width, tile_height,
+            float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
+            _ptr(grad_opacities), _stream(vertices)), "tg_render_backward")
+    return grad_vertices, grad_colors, grad_opacities

@@ -1,0 +1,441 @@
+// tg_backward.hip -- backward of the tile compositor, one workgroup per tile.
+//
+// Fragments are visited in exact reverse blend order; the transmittance in front
+// of a fragment is reconstructed by dividing the running value by (1 - opacity),
+// as the reference does (render.cu:492).
+//
+// per_pixel_sort = 0: all pixels of a tile share the list order, so the tile's
+//   list is walked backwards in LDS-staged batches.  Each fragment yields 21
+//   gradient terms (3 vertices x {x, y, w, r, g, b, opacity}; the z gradient is
+//   identically zero, render.cu:531-533).  They are summed per list entry in
+//   LDS (wave-level DPP reduction when many lanes of a wave hit the same entry,
+//   LDS float atomics otherwise) and flushed with at most 21 global float
+//   atomics per (tile, entry) instead of 24 per (pixel, entry).
+// per_pixel_sort = 1: every pixel has its own order; the pixel re-selects its
+//   fragments from the far end (32 at a time, below the (depth, position) of the
+//   last blended fragment saved by the forward pass) and issues its atomics
+//   directly.
+#include "tg_raster.hpp"
+
+namespace tg {
+
+struct BackwardArgs {
+    const float4 *grad_image;
+    const float *grad_depthmap;
+    const float4 *image;
+    const float *depthmap;
+    const float *weights;
+    const int32_t *ends;
+    const int32_t *last;
+    const float *last_depth;
+    float *grad_vertices;
+    float *grad_colors;
+    float *grad_opacities;
+};
+
+// process_backward's inputs for one list entry.
+struct alignas(16) BackRecord {
+    float m[9];
+    float w[3];
+    float iw[3];
+    float op[3];
+    float col[9];
+    float xy[6];  // ax, ay, bx, by, cx, cy
+    int id[3];
+};
+static_assert(sizeof(BackRecord) == 144, "BackRecord layout");
+
+__device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackRecord &r) {
+    const TriIds t = load_ids(a, j);
+    const float *m = a.bary + 9 * (int64_t)t.tri;
+#pragma unroll
+    for (int k = 0; k < 9; k++) r.m[k] = m[k];
+    const float4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
+    r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
+    r.iw[0] = 1.0f / va.w; r.iw[1] = 1.0f / vb.w; r.iw[2] = 1.0f / vc.w;
+    r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        r.col[k] = a.colors[3 * (int64_t)t.ia + k];
+        r.col[3 + k] = a.colors[3 * (int64_t)t.ib + k];
+        r.col[6 + k] = a.colors[3 * (int64_t)t.ic + k];
+    }
+    r.xy[0] = va.x; r.xy[1] = va.y; r.xy[2] = vb.x; r.xy[3] = vb.y; r.xy[4] = vc.x; r.xy[5] = vc.y;
+    r.id[0] = t.ia; r.id[1] = t.ib; r.id[2] = t.ic;
+}
+
+// Reverse-traversal state of one pixel (render.cu:647-653).
+struct BackState {
+    float final_alpha, alpha, s0, s1, s2, oa, zoa, final_weight, final_depth;
+    float g0, g1, g2, g3, gd;  // upstream gradient of this pixel
+};
+
+constexpr int kTerms = 21;  // per vertex v: [7v+0] x, [7v+1] y, [7v+2] w, [7v+3..5] rgb, [7v+6] opacity
+
+// util.h:299-317 scalar interpolate3_backward.
+__device__ __forceinline__ void interp_backward_scalar(float g, const float b[3], const float v[3], const float w[3],
+                                                       float gb[3], float gv[3], float gw[3]) {
+    const float nom = (b[0] * w[0] * v[0] + b[1] * w[1] * v[1]) + b[2] * w[2] * v[2];
+    const float denom = (b[0] * w[0] + b[1] * w[1]) + b[2] * w[2];
+    if (denom * denom < kEffZero) {
+#pragma unroll
+        for (int k = 0; k < 3; k++) gb[k] = gv[k] = gw[k] = 0.0f;
+        return;
+    }
+    const float inv2 = 1.0f / (denom * denom);
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        gb[k] = g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
+        gv[k] = g * b[k] * w[k] / denom;
+        gw[k] = g * (b[k] * v[k] * denom - nom * b[k]) * inv2;
+    }
+}
+
+// The arithmetic of process_backward (render.cu:455-538) for a fragment known
+// to be inside; `out` receives the 21 gradient terms.
+__device__ __forceinline__ void fragment_backward(BackState &st, const BackRecord &r, float b0, float b1, float b2, float px,
+                                                  float py, float out[kTerms]) {
+    const float b[3] = {b0, b1, b2};
+    const float w[3] = {r.w[0], r.w[1], r.w[2]};
+    const float ones[3] = {1.0f, 1.0f, 1.0f};
+    float o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
+    o = clampf(o, 0.0f, kMaxOpacity);
+    float color[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) color[k] = interp_w(b0, b1, b2, r.col[k], r.col[3 + k], r.col[6 + k], w[0], w[1], w[2]);
+    const float z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+
+    const float om = 1.0f - o;
+    const float g[3] = {st.g0, st.g1, st.g2};
+    float s[3] = {st.s0, st.s1, st.s2};
+    float t3[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) t3[k] = (color[k] * st.alpha - s[k]) / om * g[k];
+    const float drgb_do = ((t3[0] + t3[1]) + t3[2]) + st.g3 * (-st.final_alpha / om);  // :491
+    st.alpha /= om;                                                                    // :492
+#pragma unroll
+    for (int k = 0; k < 3; k++) s[k] += color[k] * o * st.alpha;                       // :493
+    st.s0 = s[0]; st.s1 = s[1]; st.s2 = s[2];
+    const float ddw_do = st.alpha - st.oa / om;                                        // :494
+    const float dud_do = st.alpha * z - st.zoa / om;                                   // :495
+    st.oa = st.oa + o * st.alpha;                                                      // :496
+    st.zoa = st.zoa + z * o * st.alpha;                                                // :497
+    float dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
+    if (st.final_weight < kEffZero) dd_do = 0.0f;
+    const float d_do = drgb_do + dd_do;
+
+    float gb_o[3], gv_o[3], gw_o[3];
+    interp_backward_scalar(d_do, b, r.op, w, gb_o, gv_o, gw_o);
+
+    // vector interpolate3_backward for the colour (util.h:319-355)
+    const float ao = st.alpha * o;
+    const float gc[3] = {ao * g[0], ao * g[1], ao * g[2]};  // :510
+    float gb_c[3] = {0.f, 0.f, 0.f}, gw_c[3] = {0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f};
+    {
+        float nom[3];
+#pragma unroll
+        for (int k = 0; k < 3; k++) nom[k] = (b[0] * w[0] * r.col[k] + b[1] * w[1] * r.col[3 + k]) + b[2] * w[2] * r.col[6 + k];
+        const float denom = b[0] * w[0] + b[1] * w[1] + b[2] * w[2];
+        if (!(denom * denom < kEffZero)) {
+            const float inv2 = 1.0f / (denom * denom);
+#pragma unroll
+            for (int v = 0; v < 3; v++) {
+                float dfb[3], dfw[3];
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    const float a = r.col[3 * v + k];
+                    dfb[k] = w[v] * (a * denom - nom[k]) * inv2;
+                    dfw[k] = (b[v] * a * denom - nom[k] * b[v]) * inv2;
+                }
+                gb_c[v] = (gc[0] * dfb[0] + gc[1] * dfb[1]) + gc[2] * dfb[2];
+                gw_c[v] = (gc[0] * dfw[0] + gc[1] * dfw[1]) + gc[2] * dfw[2];
+                scale[v] = b[v] * w[v] / denom;
+            }
+        }
+    }
+
+    float dd_dz = ao * st.gd / st.final_weight;  // :517
+    if (st.final_weight < kEffZero) dd_dz = 0.0f;
+    float gb_z[3], gv_z[3], gw_z[3];
+    interp_backward_scalar(dd_dz, b, r.iw, ones, gb_z, gv_z, gw_z);
+
+    float gbary[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) gbary[k] = gb_o[k] + gb_c[k] + gb_z[k];  // :527
+
+    // util.h:405-455 barycentric_backward (vertex part)
+    const float ax = r.xy[0], ay = r.xy[1], bx = r.xy[2], by = r.xy[3], cx = r.xy[4], cy = r.xy[5];
+    float dxy[3][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    {
+        const float T = (bx - ax) * (cy - ay) - (by - ay) * (cx - ax);
+        const float l0 = ((bx - px) * (cy - py) - (by - py) * (cx - px)) / T;
+        const float l1 = ((cx - px) * (ay - py) - (cy - py) * (ax - px)) / T;
+        const float l2 = ((ax - px) * (by - py) - (ay - py) * (bx - px)) / T;
+        const float d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
+        if (!(fabsf(d) < kEffZero)) {
+            float J[3][2][3];
+            J[0][0][0] = l0 * (-by + cy) / d;
+            J[0][0][1] = (-cy - l1 * (by - cy) + py) / d;
+            J[0][0][2] = (by - l2 * (by - cy) - py) / d;
+            J[0][1][0] = l0 * (bx - cx) / d;
+            J[0][1][1] = (cx + l1 * (bx - cx) - px) / d;
+            J[0][1][2] = (-bx + l2 * (bx - cx) + px) / d;
+            J[1][0][0] = (cy + l0 * (ay - cy) - py) / d;
+            J[1][0][1] = l1 * (ay - cy) / d;
+            J[1][0][2] = (-ay + l2 * (ay - cy) + py) / d;
+            J[1][1][0] = (-cx - l0 * (ax - cx) + px) / d;
+            J[1][1][1] = l1 * (-ax + cx) / d;
+            J[1][1][2] = (ax - l2 * (ax - cx) - px) / d;
+            J[2][0][0] = (-by - l0 * (ay - by) + py) / d;
+            J[2][0][1] = (ay - l1 * (ay - by) - py) / d;
+            J[2][0][2] = l2 * (-ay + by) / d;
+            J[2][1][0] = (bx + l0 * (ax - bx) - px) / d;
+            J[2][1][1] = (-ax + l1 * (ax - bx) + px) / d;
+            J[2][1][2] = l2 * (ax - bx) / d;
+#pragma unroll
+            for (int v = 0; v < 3; v++)
+#pragma unroll
+                for (int c = 0; c < 2; c++) dxy[v][c] = gbary[0] * J[v][c][0] + gbary[1] * J[v][c][1] + gbary[2] * J[v][c][2];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 3; v++) {
+        const float dd_dw = -gv_z[v] / (w[v] * w[v]);   // :523-525
+        const float dw = gw_o[v] + gw_c[v] + gw_z[v];   // :530
+        out[7 * v + 0] = dxy[v][0];
+        out[7 * v + 1] = dxy[v][1];
+        out[7 * v + 2] = dw + dd_dw;
+        out[7 * v + 3] = gc[0] * scale[v];
+        out[7 * v + 4] = gc[1] * scale[v];
+        out[7 * v + 5] = gc[2] * scale[v];
+        out[7 * v + 6] = gv_o[v];
+    }
+}
+
+__device__ __forceinline__ float *term_address(const BackwardArgs &g, int vertex_id, int c) {
+    if (c < 2) return g.grad_vertices + 4 * (int64_t)vertex_id + c;
+    if (c == 2) return g.grad_vertices + 4 * (int64_t)vertex_id + 3;
+    if (c < 6) return g.grad_colors + 3 * (int64_t)vertex_id + (c - 3);
+    return g.grad_opacities + vertex_id;
+}
+
+__device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, const PixelCoord &p) {
+    BackState st;
+    const float4 gi = g.grad_image[p.index];
+    st.g0 = gi.x; st.g1 = gi.y; st.g2 = gi.z; st.g3 = gi.w;
+    st.gd = g.grad_depthmap[p.index];
+    st.final_alpha = g.image[p.index].w;
+    st.alpha = st.final_alpha;
+    st.s0 = st.s1 = st.s2 = 0.0f;
+    st.oa = st.zoa = 0.0f;
+    st.final_weight = g.weights[p.index];
+    st.final_depth = g.depthmap[p.index];
+    return st;
+}
+
+// Sum over the 64 lanes of a wave, result valid in lane 63.
+__device__ __forceinline__ float wave_reduce_add(float v) {
+#define TG_DPP_ADD(ctrl, rows) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rows, 0xf, false))
+    TG_DPP_ADD(0x111, 0xf);  // row_shr:1
+    TG_DPP_ADD(0x112, 0xf);  // row_shr:2
+    TG_DPP_ADD(0x114, 0xf);  // row_shr:4
+    TG_DPP_ADD(0x118, 0xf);  // row_shr:8
+    TG_DPP_ADD(0x142, 0xa);  // row_bcast:15
+    TG_DPP_ADD(0x143, 0xc);  // row_bcast:31
+#undef TG_DPP_ADD
+    return v;
+}
+
+constexpr int kDenseHits = 12;  // lanes of a wave hitting one entry from which the DPP reduction pays
+
+__global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
+    __shared__ BackRecord s_rec[kBatch];
+    __shared__ float s_acc[kBatch * kTerms];
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int start = a.offsets[tile];
+    const PixelCoord p = pixel_of_thread(a);
+
+    if (tid == 0) s_last = 0;
+    __syncthreads();
+    const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
+    if (my_last > 0) atomicMax(&s_last, my_last);
+    __syncthreads();
+    const int tile_last = s_last;
+
+    BackState st;
+    if (p.valid) st = load_back_state(g, p);
+
+    for (int hi = tile_last; hi > 0; hi -= kBatch) {
+        const int lo = max(0, hi - kBatch);
+        const int nb = hi - lo;
+        __syncthreads();  // the previous batch's flush has finished
+        for (int e = tid; e < nb; e += blockDim.x) gather_back(a, start + lo + e, s_rec[e]);
+        for (int i = tid; i < nb * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
+        __syncthreads();
+        for (int e = nb - 1; e >= 0; e--) {
+            const BackRecord &r = s_rec[e];
+            bool hit = false;
+            float b0 = 0.f, b1 = 0.f, b2 = 0.f;
+            if (lo + e < my_last) {
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                hit = bary_inside(b0, b1, b2);
+            }
+            const uint64_t hits = __builtin_amdgcn_ballot_w64(hit);
+            if (hits == 0) continue;  // wave-uniform
+            float term[kTerms];
+#pragma unroll
+            for (int q = 0; q < kTerms; q++) term[q] = 0.0f;
+            if (hit) fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
+            float *acc = s_acc + e * kTerms;
+            if (__builtin_popcountll(hits) >= kDenseHits) {
+#pragma unroll
+                for (int q = 0; q < kTerms; q++) {
+                    const float sum = wave_reduce_add(term[q]);
+                    if (lane == kWave - 1) atomicAdd(acc + q, sum);
+                }
+            } else if (hit) {
+#pragma unroll
+                for (int q = 0; q < kTerms; q++) atomicAdd(acc + q, term[q]);
+            }
+        }
+        __syncthreads();
+        for (int i = tid; i < nb * kTerms; i += blockDim.x) {
+            const float v = s_acc[i];
+            if (v != 0.0f) {
+                const int e = i / kTerms, q = i - e * kTerms;
+                unsafeAtomicAdd(term_address(g, s_rec[e].id[q / 7], q % 7), v);
+            }
+        }
+    }
+}
+
+// Candidate insertion for the reverse selection: keeps the `cap` LARGEST
+// (depth, position) pairs in descending order.  Positions arrive in ascending
+// order, so a candidate whose depth equals a stored one has the larger position
+// and goes in front of it.
+__device__ __forceinline__ void topk_insert_desc(const TopK &tk, int cap, int &n, float d, int j) {
+    if (n == cap && d < tk.d(cap - 1)) return;
+    int i = (n < cap) ? n : cap - 1;
+    while (i > 0 && d >= tk.d(i - 1)) {
+        tk.d(i) = tk.d(i - 1);
+        tk.j(i) = tk.j(i - 1);
+        i--;
+    }
+    tk.d(i) = d;
+    tk.j(i) = j;
+    if (n < cap) n++;
+}
+
+__global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(RasterArgs a, BackwardArgs g) {
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    const int n_threads = blockDim.x;
+    DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
+    TopK tk;
+    tk.depth = reinterpret_cast<float *>(s_dyn + sizeof(DepthRecord) * kBatch);
+    tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
+    tk.n_threads = n_threads;
+
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int start = a.offsets[tile], end = a.offsets[tile + 1];
+    const PixelCoord p = pixel_of_thread(a);
+
+    BackState st;
+    int remaining = 0;
+    // exclusive upper bound of the fragments still to visit, in (depth, position) order
+    float bound_depth = 0.0f;
+    int bound_j = 0;
+    if (p.valid) {
+        st = load_back_state(g, p);
+        remaining = min(g.ends[p.index], a.max_layers);  // render.cu:642
+        bound_depth = g.last_depth[p.index];
+        bound_j = start + g.last[p.index];  // one past the last blended entry
+    }
+    while (true) {
+        const bool want = remaining > 0;
+        if (!__syncthreads_or(want)) break;
+        const int cap = min(kLayers, remaining);
+        int found = 0;
+        for (int batch = start; batch < end; batch += kBatch) {
+            const int nb = min(kBatch, end - batch);
+            __syncthreads();
+            for (int e = tid; e < nb; e += blockDim.x) gather_depth(a, batch + e, s_rec[e]);
+            __syncthreads();
+            if (want) {
+                for (int e = 0; e < nb; e++) {
+                    const DepthRecord &r = s_rec[e];
+                    float b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    if (!bary_inside(b0, b1, b2)) continue;
+                    const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
+                    const int j = batch + e;
+                    if (pd < bound_depth || (pd == bound_depth && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
+                }
+            }
+        }
+        if (want) {
+            for (int i = 0; i < found; i++) {
+                BackRecord r;
+                gather_back(a, tk.j(i), r);
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
+                float term[kTerms];
+                fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
+#pragma unroll
+                for (int q = 0; q < kTerms; q++)
+                    if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+            }
+            if (found < cap) {
+                remaining = 0;  // list exhausted
+            } else {
+                remaining -= found;
+                bound_depth = tk.d(found - 1);
+                bound_j = tk.j(found - 1);
+            }
+        }
+    }
+}
+
+}  // namespace tg
+
+using namespace tg;
+
+extern "C" int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
+                                  const int32_t *indices, const float *colors, const float *opacities,
+                                  const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
+                                  const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
+                                  const float *last_depth, int width, int height, int tile_w, int tile_h,
+                                  float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
+                                  float *grad_colors, float *grad_opacities, void *stream) {
+    if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
+    if (!grad_image || !grad_depthmap || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
+        !depthmap || !final_weights || !ends || !last || !grad_vertices || !grad_colors || !grad_opacities ||
+        (per_pixel_sort && !last_depth)) {
+        set_error("tg_render_backward: null pointer");
+        return TG_E_ARG;
+    }
+    if (((uintptr_t)vertices & 15) || ((uintptr_t)image & 15) || ((uintptr_t)grad_image & 15)) {
+        set_error("tg_render_backward: vertices, image and grad_image must be 16-byte aligned");
+        return TG_E_ARG;
+    }
+    RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+                 width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
+    BackwardArgs g{(const float4 *)grad_image, grad_depthmap, (const float4 *)image, depthmap, final_weights, ends, last,
+                   last_depth, grad_vertices, grad_colors, grad_opacities};
+    hipStream_t s = (hipStream_t)stream;
+    if (!per_pixel_sort) {
+        const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
+        hipLaunchKernelGGL(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
+        return check_launch("backward_tile_order_kernel");
+    }
+    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads());
+    const size_t lds = pixel_order_lds_bytes(tl.threads);
+    static size_t lds_reserved = 0;
+    if (int e = reserve_lds("tg_render_backward", (const void *)backward_pixel_order_kernel, lds, &lds_reserved)) return e;
+    hipLaunchKernelGGL(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds, s, a, g);
+    return check_launch("backward_pixel_order_kernel");
+}

@@ -1,0 +1,237 @@
+// tg_binning.hip -- tile binning (count, key emission), tile ranges and bary matrices.
+//
+// All four kernels are HBM-bound streaming kernels:
+//   count   reads 12 B indices + 3 x 16 B vertex gathers, writes 4 B per triangle
+//   emit    one thread per KEY (not per triangle), so a triangle that covers
+//           thousands of tiles is spread over thousands of lanes; reads the
+//           triangle again (L2 hits for neighbouring keys), writes 8 B key +
+//           4 B payload per key, coalesced
+//   ranges  reads 8 B per sorted key, writes 4 B per tile
+//   bary    reads 60 B, writes 36 B per triangle
+#include "tg_common.hpp"
+
+namespace tg {
+
+constexpr int kBinThreads = 256;
+
+struct TriXYZ { float ax, ay, az, bx, by, bz, cx, cy, cz; bool ok; };
+
+// A triangle that names a vertex outside [0, n_vertices) is treated as
+// degenerate (all coordinates zero) instead of being dereferenced.
+__device__ __forceinline__ TriXYZ load_triangle(const float4 *__restrict__ vertices, int n_vertices,
+                                                const int32_t *__restrict__ indices, int t) {
+    const int ia = indices[3 * (int64_t)t], ib = indices[3 * (int64_t)t + 1], ic = indices[3 * (int64_t)t + 2];
+    TriXYZ r;
+    r.ok = (unsigned)ia < (unsigned)n_vertices && (unsigned)ib < (unsigned)n_vertices && (unsigned)ic < (unsigned)n_vertices;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 a = r.ok ? vertices[ia] : zero, b = r.ok ? vertices[ib] : zero, c = r.ok ? vertices[ic] : zero;
+    r.ax = a.x; r.ay = a.y; r.az = a.z;
+    r.bx = b.x; r.by = b.y; r.bz = b.z;
+    r.cx = c.x; r.cy = c.y; r.cz = c.z;
+    return r;
+}
+
+__global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const float4 *__restrict__ vertices, int n_vertices,
+                                                                const int32_t *__restrict__ indices, int n_triangles, int W,
+                                                                int H, int tw, int th, int tiles_x, int tiles_y,
+                                                                uint32_t *__restrict__ tri_counts) {
+    const int t = blockIdx.x * kBinThreads + threadIdx.x;
+    if (t >= n_triangles) return;
+    const TriXYZ p = load_triangle(vertices, n_vertices, indices, t);
+    const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
+    tri_counts[t] = rect_count(r);
+}
+
+// Per-thread polygon storage in LDS, slot-major so that lanes never conflict.
+constexpr int kPolyCap = 8;
+struct PolyLds {
+    float x[2][kPolyCap][kBinThreads];
+    float y[2][kPolyCap][kBinThreads];
+};
+
+// One Sutherland-Hodgman pass (render.cu:159-189) from buffer `src` to `1-src`
+// against nx*x + ny*y - d >= 0.  Returns the new vertex count.
+__device__ __forceinline__ int clip_pass(PolyLds &lds, int src, int n_in, float nx, float ny, float d) {
+    const int tid = threadIdx.x;
+    const int dst = 1 - src;
+    int n_out = 0;
+    float p0x = lds.x[src][n_in - 1][tid], p0y = lds.y[src][n_in - 1][tid];
+    float d0 = nx * p0x + ny * p0y - d;
+    bool in0 = d0 >= 0.0f;
+    for (int i = 0; i < n_in; i++) {
+        const float p1x = lds.x[src][i][tid], p1y = lds.y[src][i][tid];
+        const float d1 = nx * p1x + ny * p1y - d;
+        const bool in1 = d1 >= 0.0f;
+        // A convex polygon gains at most one vertex per pass (7 after four); the
+        // capacity test only matters for slivers whose in/out pattern alternates
+        // by rounding, where vertices beyond the eighth are dropped.
+        if (in1 != in0 && n_out < kPolyCap) {
+            const float t = d0 / (d0 - d1);
+            lds.x[dst][n_out][tid] = p0x + t * (p1x - p0x);
+            lds.y[dst][n_out][tid] = p0y + t * (p1y - p0y);
+            n_out++;
+        }
+        if (in1 && n_out < kPolyCap) {
+            lds.x[dst][n_out][tid] = p1x;
+            lds.y[dst][n_out][tid] = p1y;
+            n_out++;
+        }
+        p0x = p1x; p0y = p1y; d0 = d1; in0 = in1;
+    }
+    return n_out;
+}
+
+// Index of the triangle that owns key k: the last i with tri_offsets[i] <= k.
+__device__ __forceinline__ int owner_of_key(const uint32_t *__restrict__ tri_offsets, int n_triangles, uint32_t k) {
+    int lo = 0, hi = n_triangles;  // invariant: tri_offsets[lo] <= k, answer in [lo, hi)
+    while (hi - lo > 1) {
+        const int mid = lo + ((hi - lo) >> 1);
+        if (tri_offsets[mid] <= k) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__restrict__ vertices, int n_vertices,
+                                                               const int32_t *__restrict__ indices, int n_triangles, int W,
+                                                               int H, int tw, int th, int tiles_x, int tiles_y,
+                                                               const uint32_t *__restrict__ tri_offsets, int64_t n_keys,
+                                                               uint64_t *__restrict__ keys, uint32_t *__restrict__ payload) {
+    __shared__ PolyLds lds;
+    const int tid = threadIdx.x;
+    const int64_t k = (int64_t)blockIdx.x * kBinThreads + tid;
+    if (k >= n_keys) return;  // no barrier below: the LDS arrays are private per thread
+
+    const int t = owner_of_key(tri_offsets, n_triangles, (uint32_t)k);
+    const uint32_t local = (uint32_t)k - tri_offsets[t];
+    const TriXYZ p = load_triangle(vertices, n_vertices, indices, t);
+    const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
+    const uint32_t ny = (uint32_t)(r.y1 - r.y0 + 1);
+    const int tx = r.x0 + (int)(local / ny);  // tile x outer, tile y inner (render.cu:235-236)
+    const int ty = r.y0 + (int)(local % ny);
+
+    // render.cu:140-152 compute_plane
+    const float det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+    const float id = (float)(1.0 / (double)det);
+    const float A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
+    const float B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
+    const float C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
+
+    // render.cu:243-246 tile rectangle in NDC
+    const float xmin = (float)(tx * tw) / (float)W * 2.0f - 1.0f;
+    const float xmax = (float)((tx + 1) * tw) / (float)W * 2.0f - 1.0f;
+    const float ymin = (float)(ty * th) / (float)H * 2.0f - 1.0f;
+    const float ymax = (float)((ty + 1) * th) / (float)H * 2.0f - 1.0f;
+
+    lds.x[0][0][tid] = p.ax; lds.y[0][0][tid] = p.ay;
+    lds.x[0][1][tid] = p.bx; lds.y[0][1][tid] = p.by;
+    lds.x[0][2][tid] = p.cx; lds.y[0][2][tid] = p.cy;
+    int n = 3;
+    n = clip_pass(lds, 0, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
+    if (n > 0) n = clip_pass(lds, 1, n, -1.0f, 0.0f, -xmax);
+    if (n > 0) n = clip_pass(lds, 0, n, 0.0f, 1.0f, ymin);
+    if (n > 0) n = clip_pass(lds, 1, n, 0.0f, -1.0f, -ymax);
+
+    float key = kFarKey;  // render.cu:259
+    if (n > 0) {
+        float md = FLT_MAX;
+        for (int i = 0; i < n; i++) {
+            const float pd = A * lds.x[0][i][tid] + B * lds.y[0][i][tid] + C;  // render.cu:154-157
+            md = (pd < md) ? pd : md;
+        }
+        key = md;
+    }
+    const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
+    keys[k] = ((uint64_t)tile << 32) | orderable_bits(key);
+    payload[k] = (uint32_t)t;
+}
+
+__global__ __launch_bounds__(kBinThreads) void tile_ranges_kernel(const uint64_t *__restrict__ sorted_keys, int64_t n_keys,
+                                                                  int n_tiles, int32_t *__restrict__ offsets) {
+    const int64_t i = (int64_t)blockIdx.x * kBinThreads + threadIdx.x;
+    if (i > n_keys) return;
+    const int cur = (i < n_keys) ? (int)(sorted_keys[i] >> 32) : n_tiles;
+    const int prev = (i > 0) ? (int)(sorted_keys[i - 1] >> 32) : -1;
+    for (int t = prev + 1; t <= cur && t <= n_tiles; t++) offsets[t] = (int32_t)i;
+}
+
+// render.cu:310-337 cartesian_to_bary_kernel.
+__global__ __launch_bounds__(kBinThreads) void bary_kernel(const float4 *__restrict__ vertices, int n_vertices,
+                                                           const int32_t *__restrict__ indices, int n_triangles,
+                                                           float *__restrict__ out) {
+    const int t = blockIdx.x * kBinThreads + threadIdx.x;
+    if (t >= n_triangles) return;
+    const TriXYZ p = load_triangle(vertices, n_vertices, indices, t);
+    float denom = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+    if (fabsf(denom) < kEffZero) denom = 1.0f;
+    float *m = out + 9 * (int64_t)t;
+    m[0] = (p.by - p.cy) / denom;
+    m[1] = (p.cx - p.bx) / denom;
+    m[2] = (p.bx * p.cy - p.cx * p.by) / denom;
+    m[3] = (p.cy - p.ay) / denom;
+    m[4] = (p.ax - p.cx) / denom;
+    m[5] = (p.cx * p.ay - p.ax * p.cy) / denom;
+    m[6] = (p.ay - p.by) / denom;
+    m[7] = (p.bx - p.ax) / denom;
+    m[8] = (p.ax * p.by - p.bx * p.ay) / denom;
+}
+
+static int check_geometry(const char *fn, const void *vertices, int n_vertices, const void *indices, int n_triangles, int W, int H,
+                          int tw, int th) {
+    if (n_triangles < 0 || n_vertices < 0 || W <= 0 || H <= 0 || tw <= 0 || th <= 0 || (n_triangles > 0 && (!vertices || !indices))) {
+        set_error("%s: null pointer, negative count or non-positive image/tile size", fn);
+        return TG_E_ARG;
+    }
+    if ((uintptr_t)vertices & 15) {
+        set_error("%s: vertices must be 16-byte aligned", fn);
+        return TG_E_ARG;
+    }
+    return 0;
+}
+
+}  // namespace tg
+
+using namespace tg;
+
+extern "C" int tg_bin_count(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+                            int tile_h, uint32_t *tri_counts, void *stream) {
+    if (int e = check_geometry("tg_bin_count", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
+    if (n_triangles == 0) return 0;
+    if (!tri_counts) { set_error("tg_bin_count: tri_counts is null"); return TG_E_ARG; }
+    hipLaunchKernelGGL(bin_count_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+                       (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
+                       ceil_div(width, tile_w), ceil_div(height, tile_h), tri_counts);
+    return check_launch("bin_count_kernel");
+}
+
+extern "C" int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+                           int tile_h, const uint32_t *tri_offsets, int64_t n_keys, uint64_t *keys, uint32_t *payload,
+                           void *stream) {
+    if (int e = check_geometry("tg_bin_emit", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
+    if (n_keys < 0 || n_keys > 0xffffffffll) { set_error("tg_bin_emit: n_keys out of range"); return TG_E_ARG; }
+    if (n_keys == 0) return 0;
+    if (n_triangles == 0 || !tri_offsets || !keys || !payload) { set_error("tg_bin_emit: null pointer"); return TG_E_ARG; }
+    hipLaunchKernelGGL(bin_emit_kernel, dim3((unsigned)ceil_div64(n_keys, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+                       (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
+                       ceil_div(width, tile_w), ceil_div(height, tile_h), tri_offsets, n_keys, keys, payload);
+    return check_launch("bin_emit_kernel");
+}
+
+extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int32_t *offsets, void *stream) {
+    if (n_keys < 0 || n_keys > 0x7fffffffll || n_tiles <= 0 || !offsets || (n_keys > 0 && !sorted_keys)) {
+        set_error("tg_tile_ranges: null pointer or size out of range");
+        return TG_E_ARG;
+    }
+    hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)ceil_div64(n_keys + 1, kBinThreads)), dim3(kBinThreads), 0,
+                       (hipStream_t)stream, sorted_keys, n_keys, n_tiles, offsets);
+    return check_launch("tile_ranges_kernel");
+}
+
+extern "C" int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, float *out,
+                       void *stream) {
+    if (int e = check_geometry("tg_bary", vertices, n_vertices, indices, n_triangles, 1, 1, 1, 1)) return e;
+    if (n_triangles == 0) return 0;
+    if (!out) { set_error("tg_bary: out is null"); return TG_E_ARG; }
+    hipLaunchKernelGGL(bary_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+                       (const float4 *)vertices, n_vertices, indices, n_triangles, out);
+    return check_launch("bary_kernel");
+}

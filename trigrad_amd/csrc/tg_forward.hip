@@ -1,0 +1,245 @@
+// tg_forward.hip -- forward rasterize-and-blend, one workgroup per tile.
+//
+// per_pixel_sort = 0 (tile order): the sorted tile list is staged into LDS in
+//   batches of 256 records; each pixel composites front to back and stops as
+//   soon as its transmittance falls to the threshold or max_layers fragments
+//   are blended; the workgroup leaves the list when every pixel has stopped.
+// per_pixel_sort = 1: each pixel repeatedly selects its next (up to 32) nearest
+//   fragments in (pixel depth, list position) order by scanning the whole list
+//   (records staged through LDS as above, candidate lists in LDS, slot-major),
+//   then blends them; threshold and max_layers are tested between selections
+//   only, as in the reference (render.cu:588).
+//
+// Not HBM-bound: per (pixel, entry) pair ~12 VALU operations and three
+// broadcast LDS reads against 148 B of gathered data per ENTRY.
+#include "tg_raster.hpp"
+
+namespace tg {
+
+struct ForwardOut {
+    float4 *image;
+    float *depthmap;
+    float *weights;
+    int32_t *ends;
+    int32_t *last;
+    float *last_depth;
+};
+
+__device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, float last_depth) {
+    // render.cu:609-618
+    float depth;
+    if (s.weight > kEffZero) {
+        depth = s.depth / s.weight;
+    } else {
+        depth = __builtin_inff();
+        s.weight = 0.0f;
+    }
+    o.depthmap[p.index] = depth;
+    o.weights[p.index] = s.weight;
+    o.ends[p.index] = s.blended;
+    if (o.last) o.last[p.index] = last;
+    if (o.last_depth) o.last_depth[p.index] = last_depth;
+    o.image[p.index] = make_float4(s.c0, s.c1, s.c2, s.alpha);
+}
+
+__global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(RasterArgs a, ForwardOut out) {
+    __shared__ BlendRecord s_rec[kBatch];
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int start = a.offsets[tile], end = a.offsets[tile + 1];
+    const PixelCoord p = pixel_of_thread(a);
+
+    PixelState s;
+    int last = 0;
+    for (int batch = start; batch < end; batch += kBatch) {
+        const bool running = p.valid && s.alpha > a.thr && s.blended < a.max_layers;
+        if (!__syncthreads_or(running)) break;
+        const int nb = min(kBatch, end - batch);
+        for (int e = tid; e < nb; e += blockDim.x) gather_blend(a, batch + e, s_rec[e]);
+        __syncthreads();
+        if (running) {
+            for (int e = 0; e < nb; e++) {
+                if (!(s.alpha > a.thr && s.blended < a.max_layers)) break;  // render.cu:578
+                const BlendRecord &r = s_rec[e];
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                if (!bary_inside(b0, b1, b2)) continue;
+                blend_fragment(s, r, b0, b1, b2);
+                last = batch + e - start + 1;
+            }
+        }
+    }
+    if (p.valid) write_pixel(out, p, s, last, 0.0f);
+}
+
+// render.cu:338-373 insert_sorted_topk on an LDS candidate list of capacity `cap`.
+__device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, float d, int j) {
+    if (n == cap && d >= tk.d(cap - 1)) return;
+    int i = (n < cap) ? n : cap - 1;
+    while (i > 0 && d < tk.d(i - 1)) {
+        tk.d(i) = tk.d(i - 1);
+        tk.j(i) = tk.j(i - 1);
+        i--;
+    }
+    tk.d(i) = d;
+    tk.j(i) = j;
+    if (n < cap) n++;
+}
+
+__global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(RasterArgs a, ForwardOut out) {
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    const int n_threads = blockDim.x;
+    DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
+    TopK tk;
+    tk.depth = reinterpret_cast<float *>(s_dyn + sizeof(DepthRecord) * kBatch);
+    tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
+    tk.n_threads = n_threads;
+
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int start = a.offsets[tile], end = a.offsets[tile + 1];
+    const PixelCoord p = pixel_of_thread(a);
+
+    PixelState s;
+    float last_depth = -__builtin_inff();  // render.cu:585-586
+    int last_j = -1;
+    bool active = p.valid;
+    while (true) {
+        const bool want = active && s.alpha > a.thr && s.blended < a.max_layers;  // render.cu:588
+        if (!__syncthreads_or(want)) break;
+        const int cap = want ? min(kLayers, a.max_layers - s.blended) : 0;
+        int found = 0;
+        for (int batch = start; batch < end; batch += kBatch) {
+            const int nb = min(kBatch, end - batch);
+            __syncthreads();
+            for (int e = tid; e < nb; e += blockDim.x) gather_depth(a, batch + e, s_rec[e]);
+            __syncthreads();
+            if (want) {
+                for (int e = 0; e < nb; e++) {
+                    const DepthRecord &r = s_rec[e];
+                    float b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    if (!bary_inside(b0, b1, b2)) continue;
+                    const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
+                    const int j = batch + e;
+                    if (pd < last_depth) continue;
+                    if (pd == last_depth && j <= last_j) continue;
+                    topk_insert(tk, cap, found, pd, j);
+                }
+            }
+        }
+        if (want) {
+            if (found == 0) {
+                active = false;  // render.cu:594
+            } else {
+                const int todo = min(found, a.max_layers - s.blended);
+                for (int i = 0; i < todo; i++) {
+                    BlendRecord r;
+                    gather_blend(a, tk.j(i), r);
+                    float b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
+                    blend_fragment(s, r, b0, b1, b2);
+                }
+                last_depth = tk.d(todo - 1);
+                last_j = tk.j(todo - 1);
+                // fewer candidates than asked for: the list is exhausted, the next
+                // selection would return nothing (render.cu:594)
+                if (found < cap) active = false;
+            }
+        }
+    }
+    if (p.valid) write_pixel(out, p, s, last_j >= 0 ? last_j - start + 1 : 0, last_depth);
+}
+
+TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads) {
+    TileLaunch t;
+    const int pixels = tile_w * tile_h;
+    t.threads = min(ceil_div(pixels, kWave) * kWave, max_threads);
+    t.grid = dim3(ceil_div(width, tile_w), ceil_div(height, tile_h), ceil_div(pixels, t.threads));
+    return t;
+}
+
+// Workgroup size of the per-pixel-sort kernels.  Their candidate lists take
+// 32 * 8 bytes of LDS per thread; 256 threads need 80 KB in one workgroup,
+// which gfx950 (160 KB LDS) provides.  TRIGRAD_PIXEL_ORDER_THREADS overrides.
+int pixel_order_threads() {
+    static int cached = 0;
+    if (!cached) {
+        int v = kTileThreads;
+        if (const char *e = getenv("TRIGRAD_PIXEL_ORDER_THREADS")) {
+            const int x = atoi(e);
+            if (x == 64 || x == 128 || x == 256) v = x;
+        }
+        cached = v;
+    }
+    return cached;
+}
+
+size_t pixel_order_lds_bytes(int n_threads) {
+    return sizeof(DepthRecord) * kBatch + (size_t)kLayers * n_threads * (sizeof(float) + sizeof(int));
+}
+
+// Dynamic LDS beyond 64 KB has to be enabled per kernel once.
+int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved) {
+    if (bytes <= 64 * 1024 || bytes <= *reserved) return 0;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        set_error("%s: cannot reserve %zu bytes of LDS per workgroup: %s", fn, bytes, hipGetErrorString(e));
+        return (int)e;
+    }
+    *reserved = bytes;
+    return 0;
+}
+
+int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers) {
+    if (width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0 || tile_w * tile_h > kMaxTilePixels) {
+        set_error("%s: image size must be positive and tile_w*tile_h in [1, %d]", fn, kMaxTilePixels);
+        return TG_E_ARG;
+    }
+    if ((int64_t)width * height > 0x7fffffffll) {
+        set_error("%s: image too large", fn);
+        return TG_E_ARG;
+    }
+    if (max_layers <= 0) {
+        set_error("%s: max_layers must be positive", fn);
+        return TG_E_ARG;
+    }
+    return 0;
+}
+
+}  // namespace tg
+
+using namespace tg;
+
+extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, const float *colors, const float *opacities,
+                                 const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
+                                 int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
+                                 float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
+                                 float *last_depth, void *stream) {
+    if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
+    if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
+        set_error("tg_render_forward: null pointer");
+        return TG_E_ARG;
+    }
+    if (((uintptr_t)vertices & 15) || ((uintptr_t)image & 15)) {
+        set_error("tg_render_forward: vertices and image must be 16-byte aligned");
+        return TG_E_ARG;
+    }
+    RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+                 width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
+    ForwardOut o{(float4 *)image, depthmap, final_weights, ends, last, last_depth};
+    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads() : kTileThreads);
+    const dim3 grid = tl.grid;
+    const int n_threads = tl.threads;
+    hipStream_t s = (hipStream_t)stream;
+    if (!per_pixel_sort) {
+        hipLaunchKernelGGL(forward_tile_order_kernel, grid, dim3(n_threads), 0, s, a, o);
+        return check_launch("forward_tile_order_kernel");
+    }
+    const size_t lds = pixel_order_lds_bytes(n_threads);
+    static size_t lds_reserved = 0;
+    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel, lds, &lds_reserved)) return e;
+    hipLaunchKernelGGL(forward_pixel_order_kernel, grid, dim3(n_threads), lds, s, a, o);
+    return check_launch("forward_pixel_order_kernel");
+}

@@ -1,0 +1,153 @@
+// tg_raster.hpp -- pieces shared by the forward and backward tile kernels.
+//
+// Launch shape: grid (tiles_x, tiles_y, parts); a workgroup of at most 256 threads
+// owns pixels [z*blockDim, (z+1)*blockDim) of its tile in row-major order, so a
+// 16x16 tile is exactly one workgroup of four waves and larger tiles are split
+// into several workgroups that walk the same list.  A tile's sorted list is consumed in
+// batches: up to kBatch threads each gather one list entry (triangle id ->
+// vertex ids -> vertex data, bary matrix, attributes) into an LDS record, then
+// every pixel thread walks the records; all lanes read the same record at the
+// same time, which LDS serves as a broadcast.
+#pragma once
+#include "tg_common.hpp"
+
+namespace tg {
+
+constexpr int kBatch = 256;         // list entries staged per batch
+constexpr int kLayers = 32;         // per-pixel selection batch (render.cu:570, :655)
+constexpr int kMaxTilePixels = 1024;  // tile_w * tile_h limit of the API (wrapper.py:143)
+constexpr int kTileThreads = 256;     // workgroup size limit
+
+struct RasterArgs {
+    const float4 *vertices;
+    const int32_t *indices;
+    const float *colors;
+    const float *opacities;
+    const int32_t *sorted_ids;
+    const int32_t *offsets;
+    const float *bary;
+    int W, H, tw, th;
+    float thr;
+    int max_layers;
+};
+
+struct PixelCoord {
+    int ix, iy, index;
+    bool valid;
+    float px, py;
+};
+
+__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
+    PixelCoord p;
+    const int t = blockIdx.z * blockDim.x + threadIdx.x;
+    const int lx = t % a.tw, ly = t / a.tw;
+    p.ix = blockIdx.x * a.tw + lx;
+    p.iy = blockIdx.y * a.th + ly;
+    p.valid = (t < a.tw * a.th) && p.ix < a.W && p.iy < a.H;  // render.cu:554
+    p.index = p.iy * a.W + p.ix;
+    p.px = pixel_ndc(p.ix, a.W);
+    p.py = pixel_ndc(p.iy, a.H);
+    return p;
+}
+
+// Everything process_forward (render.cu:417-453) reads for one list entry.
+struct alignas(16) BlendRecord {
+    float m[9];
+    float w[3];
+    float iw[3];   // 1/w per vertex (render.cu:444)
+    float op[3];
+    float col[9];  // vertex a rgb, vertex b rgb, vertex c rgb
+    float pad;
+};
+static_assert(sizeof(BlendRecord) == 112, "BlendRecord layout");
+
+// What select_next_k_in_tile (render.cu:375-415) reads for one list entry.
+struct alignas(16) DepthRecord {
+    float m[9];
+    float z[3];
+    float w[3];
+    float pad;
+};
+static_assert(sizeof(DepthRecord) == 64, "DepthRecord layout");
+
+struct TriIds { int tri, ia, ib, ic; };
+
+__device__ __forceinline__ TriIds load_ids(const RasterArgs &a, int j) {
+    TriIds t;
+    t.tri = a.sorted_ids[j];
+    t.ia = a.indices[3 * (int64_t)t.tri];
+    t.ib = a.indices[3 * (int64_t)t.tri + 1];
+    t.ic = a.indices[3 * (int64_t)t.tri + 2];
+    return t;
+}
+
+__device__ __forceinline__ void gather_blend(const RasterArgs &a, int j, BlendRecord &r) {
+    const TriIds t = load_ids(a, j);
+    const float *m = a.bary + 9 * (int64_t)t.tri;
+#pragma unroll
+    for (int k = 0; k < 9; k++) r.m[k] = m[k];
+    const float wa = a.vertices[t.ia].w, wb = a.vertices[t.ib].w, wc = a.vertices[t.ic].w;
+    r.w[0] = wa; r.w[1] = wb; r.w[2] = wc;
+    r.iw[0] = 1.0f / wa; r.iw[1] = 1.0f / wb; r.iw[2] = 1.0f / wc;
+    r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        r.col[k] = a.colors[3 * (int64_t)t.ia + k];
+        r.col[3 + k] = a.colors[3 * (int64_t)t.ib + k];
+        r.col[6 + k] = a.colors[3 * (int64_t)t.ic + k];
+    }
+}
+
+__device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRecord &r) {
+    const TriIds t = load_ids(a, j);
+    const float *m = a.bary + 9 * (int64_t)t.tri;
+#pragma unroll
+    for (int k = 0; k < 9; k++) r.m[k] = m[k];
+    const float4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
+    r.z[0] = va.z; r.z[1] = vb.z; r.z[2] = vc.z;
+    r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
+}
+
+// Front-to-back compositing state of one pixel (render.cu:564-574).
+struct PixelState {
+    float alpha = 1.0f, c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, depth = 0.0f, weight = 0.0f;
+    int blended = 0;
+};
+
+// The arithmetic of process_forward for a fragment known to be inside.
+__device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord &r, float b0, float b1, float b2) {
+    float o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], r.w[0], r.w[1], r.w[2]);
+    o = clampf(o, 0.0f, kMaxOpacity);
+    const float k0 = interp_w(b0, b1, b2, r.col[0], r.col[3], r.col[6], r.w[0], r.w[1], r.w[2]);
+    const float k1 = interp_w(b0, b1, b2, r.col[1], r.col[4], r.col[7], r.w[0], r.w[1], r.w[2]);
+    const float k2 = interp_w(b0, b1, b2, r.col[2], r.col[5], r.col[8], r.w[0], r.w[1], r.w[2]);
+    const float z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+    const float ao = s.alpha * o;
+    s.depth = s.depth + ao * z;
+    s.weight = s.weight + ao;
+    s.c0 = s.c0 + ao * k0;
+    s.c1 = s.c1 + ao * k1;
+    s.c2 = s.c2 + ao * k2;
+    s.alpha *= (1.0f - o);
+    s.blended++;
+}
+
+// ---- host-side launch helpers (defined in tg_forward.hip) ---------------------------
+struct TileLaunch { dim3 grid; int threads; };
+TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads);
+int pixel_order_threads();
+size_t pixel_order_lds_bytes(int n_threads);
+int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
+int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
+
+// Per-pixel candidate lists of the per-pixel-sort mode live in LDS, slot-major:
+// entry `slot` of thread `t` is at [slot * n_threads + t] (conflict-free).
+struct TopK {
+    float *depth;
+    int *pos;
+    int n_threads;
+    __device__ __forceinline__ float &d(int slot) const { return depth[slot * n_threads + threadIdx.x]; }
+    __device__ __forceinline__ int &j(int slot) const { return pos[slot * n_threads + threadIdx.x]; }
+};
+
+}  // namespace tg

@@ -1,0 +1,182 @@
+// tg_scan.hip -- single-pass exclusive prefix sum of uint32 with decoupled look-back.
+//
+// HBM-bound: 4 B read + 4 B written per element, one pass.  A workgroup of
+// 512 threads owns a tile of 2048 elements (one 16-byte load per thread).
+// Inside a wave the scan runs on DPP row shifts and row broadcasts (wave64);
+// the tile prefix comes from the predecessors' published state words, read by
+// one wave, 64 predecessors per step.
+//
+// State word (one uint64 per tile): bits 63..62 = 0 not ready, 1 tile aggregate
+// ready, 2 inclusive prefix ready; bits 31..0 = the value.  Value and flag
+// share one word, so relaxed agent-scope atomic loads/stores are sufficient.
+// Tiles are numbered by an atomic ticket taken at workgroup start, so every
+// tile a workgroup waits for is already running.  The wait is bounded: on
+// expiry the kernel records TG_STATUS_LOOKBACK_TIMEOUT and carries on (with a
+// wrong result) so that every wave still exits.
+#include "tg_common.hpp"
+
+namespace tg {
+
+constexpr int kScanThreads = 512;
+constexpr int kScanTile = kScanThreads * 4;
+constexpr uint32_t kSpinLimit = 1u << 20;
+
+constexpr uint64_t kFlagAggregate = 1ull << 62;
+constexpr uint64_t kFlagInclusive = 2ull << 62;
+
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ uint32_t dpp_add(uint32_t v) {
+    // lanes whose source is out of range (or whose row is masked off) receive 0
+    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false);
+}
+
+// Inclusive scan over the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+    v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+    v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+    v = dpp_add<0x118, 0xf>(v);  // row_shr:8
+    v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+    v = wave_inclusive_scan(v);
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+__global__ void scan_init_kernel(uint32_t *ticket, uint64_t *states, int n_tiles, uint32_t *total, uint32_t *status) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i == 0) {
+        *ticket = 0;
+        *total = 0;
+        if (status) *status = TG_STATUS_OK;
+    }
+    if (i < n_tiles) states[i] = 0;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint32_t *__restrict__ in, uint32_t *out, int64_t n,
+                                                                     uint32_t *total, uint32_t *ticket, uint64_t *states,
+                                                                     int n_tiles, uint32_t *status) {
+    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_wave_total[kScanThreads / kWave];
+    __shared__ uint32_t s_tile_prefix;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    __syncthreads();
+    const int tile = (int)s_tile;
+
+    const int64_t base = (int64_t)tile * kScanTile + (int64_t)tid * 4;
+    uint32_t x[4] = {0, 0, 0, 0};
+    if (base + 4 <= n) {
+        uint4 v = *reinterpret_cast<const uint4 *>(in + base);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else {
+        for (int k = 0; k < 4; k++)
+            if (base + k < n) x[k] = in[base + k];
+    }
+    const uint32_t thread_sum = x[0] + x[1] + x[2] + x[3];
+    const uint32_t incl = wave_inclusive_scan(thread_sum);
+    if (lane == kWave - 1) s_wave_total[wave] = incl;
+    __syncthreads();
+
+    if (wave == 0) {
+        // scan of the wave totals, then publish and look back
+        uint32_t wt = (lane < kScanThreads / kWave) ? s_wave_total[lane] : 0u;
+        uint32_t wincl = wave_inclusive_scan(wt);
+        uint32_t tile_total = (uint32_t)__builtin_amdgcn_readlane((int)wincl, kScanThreads / kWave - 1);
+        if (lane < kScanThreads / kWave) s_wave_total[lane] = wincl - wt;  // exclusive wave offsets
+
+        if (lane == 0) {
+            uint64_t word = (tile == 0 ? kFlagInclusive : kFlagAggregate) | tile_total;
+            __hip_atomic_store(&states[tile], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        uint32_t prefix = 0;
+        bool timed_out = false;
+        for (int look = tile - 1; look >= 0; look -= kWave) {
+            const int idx = look - lane;
+            uint64_t word = kFlagInclusive;  // before the first tile: inclusive prefix 0
+            if (idx >= 0) {
+                uint32_t spins = 0;
+                word = __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                while ((word >> 62) == 0 && spins < kSpinLimit) {
+                    __builtin_amdgcn_s_sleep(1);
+                    word = __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    spins++;
+                }
+                if ((word >> 62) == 0) timed_out = true;
+            }
+            const uint64_t inclusive_lanes = __builtin_amdgcn_ballot_w64((word >> 62) == 2);
+            const int first = inclusive_lanes ? __builtin_ctzll(inclusive_lanes) : kWave;
+            prefix += wave_sum(lane <= first ? (uint32_t)word : 0u);
+            if (inclusive_lanes) break;
+        }
+        if (__builtin_amdgcn_ballot_w64(timed_out) && lane == 0 && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
+        if (lane == 0) {
+            if (tile != 0)
+                __hip_atomic_store(&states[tile], kFlagInclusive | (uint64_t)(prefix + tile_total), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            s_tile_prefix = prefix;
+            if (tile == n_tiles - 1) *total = prefix + tile_total;
+        }
+    }
+    __syncthreads();
+
+    uint32_t run = s_tile_prefix + s_wave_total[wave] + (incl - thread_sum);
+    uint32_t y[4];
+    for (int k = 0; k < 4; k++) { y[k] = run; run += x[k]; }
+    if (base + 4 <= n) {
+        *reinterpret_cast<uint4 *>(out + base) = make_uint4(y[0], y[1], y[2], y[3]);
+    } else {
+        for (int k = 0; k < 4; k++)
+            if (base + k < n) out[base + k] = y[k];
+    }
+}
+
+}  // namespace tg
+
+using namespace tg;
+
+static size_t scan_state_offset() { return 64; }  // ticket lives in the first 64 bytes
+
+extern "C" size_t tg_scan_workspace_bytes(int64_t n) {
+    if (n < 0) return 0;
+    int64_t tiles = ceil_div64(n, kScanTile);
+    if (tiles < 1) tiles = 1;
+    return scan_state_offset() + (size_t)tiles * sizeof(uint64_t);
+}
+
+extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
+                                     size_t workspace_bytes, uint32_t *status, void *stream) {
+    if (n < 0 || !total || !workspace || (n > 0 && (!in || !out))) {
+        set_error("tg_scan_exclusive_u32: null pointer or negative size");
+        return TG_E_ARG;
+    }
+    if (((uintptr_t)in & 15) || ((uintptr_t)out & 15) || ((uintptr_t)workspace & 7)) {
+        set_error("tg_scan_exclusive_u32: in/out must be 16-byte aligned, workspace 8-byte aligned");
+        return TG_E_ARG;
+    }
+    if (n > (int64_t)kScanTile * 0x7fffffff / 2) {
+        set_error("tg_scan_exclusive_u32: n too large");
+        return TG_E_ARG;
+    }
+    if (workspace_bytes < tg_scan_workspace_bytes(n)) {
+        set_error("tg_scan_exclusive_u32: workspace of %zu bytes, need %zu", workspace_bytes, tg_scan_workspace_bytes(n));
+        return TG_E_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int n_tiles = (int)ceil_div64(n, kScanTile);
+    uint32_t *ticket = (uint32_t *)workspace;
+    uint64_t *states = (uint64_t *)((char *)workspace + scan_state_offset());
+    const int init_blocks = n_tiles > 0 ? ceil_div(n_tiles, 256) : 1;
+    hipLaunchKernelGGL(scan_init_kernel, dim3(init_blocks), dim3(256), 0, s, ticket, states, n_tiles, total, status);
+    if (int e = check_launch("scan_init_kernel")) return e;
+    if (n_tiles == 0) return 0;
+    hipLaunchKernelGGL(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
+                       n_tiles, status);
+    return check_launch("scan_lookback_kernel");
+}

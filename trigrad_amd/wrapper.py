@@ -1,0 +1,121 @@
+"""Public entry point: `render` and its autograd Function, with the signatures,
+defaults, checks and return values of reference src/trigrad/wrapper.py:12-158."""
+from typing import Tuple
+
+import torch
+from torch.autograd import Function
+
+from . import _C
+from .util import create_check
+
+check_tensor = create_check("cuda", _C.precision)
+precision = _C.precision
+
+
+class Renderer(Function):
+    @staticmethod
+    def forward(
+        ctx,
+        vertices: torch.Tensor,
+        indices: torch.Tensor,
+        colors: torch.Tensor,
+        opacities: torch.Tensor,
+        width: int = 500,
+        height: int = 500,
+        tile_width: int = 16,
+        tile_height: int = 16,
+        early_stopping_threshold: float = 1 / 256,
+        record_timing: bool = False,
+        per_pixel_sort: bool = True,
+        max_layers: int = 32,
+    ):
+        n_vertices, _ = vertices.shape
+        check_tensor(vertices, "vertices", (n_vertices, 4))
+        check_tensor(colors, "colors", (n_vertices, 3))
+        check_tensor(opacities, "opacities", (n_vertices,))
+        n_triangles, _ = indices.shape
+        check_tensor(indices, "indices", (n_triangles, 3), torch.int32)
+        if max_layers <= 0:
+            max_layers = n_triangles + 1  # wrapper.py:35-36: "no limit"
+
+        ctx.render_args = (width, height, tile_width, tile_height, early_stopping_threshold, per_pixel_sort, max_layers)
+        if n_triangles < 1:
+            # wrapper.py:46-53: nothing to draw -- transparent black, infinitely far
+            ctx.skipped = True
+            image = torch.zeros((height, width, 4), dtype=colors.dtype, device=colors.device)
+            image[..., 3] = 1.0
+            depthmap = torch.full((height, width), float("inf"), dtype=colors.dtype, device=colors.device)
+            timings = None
+            ctx.save_for_backward(vertices, indices, colors, opacities)
+        else:
+            ctx.skipped = False
+            (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume) = _C.render_forward(
+                vertices, indices, colors, opacities, width, height, tile_width, tile_height, early_stopping_threshold,
+                not record_timing, per_pixel_sort, max_layers)
+            last, last_depth, sort_status = resume
+            if record_timing and int(sort_status.item()) != 0:
+                raise RuntimeError("tg_sort_pairs_u64_u32: look-back wait timed out")
+            ctx.has_last_depth = last_depth is not None
+            saved = [vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, image, depthmap, final_weights,
+                     ends, last, sort_status]
+            if last_depth is not None:
+                saved.append(last_depth)
+            ctx.save_for_backward(*saved)
+        if record_timing:
+            return image, depthmap, timings
+        return image, depthmap
+
+    @staticmethod
+    def backward(ctx, grad_image, grad_depthmap, grad_timings=None):
+        if ctx.skipped:
+            grad_vertices = torch.zeros_like(ctx.saved_tensors[0])
+            grad_colors = torch.zeros_like(ctx.saved_tensors[2])
+            grad_opacities = torch.zeros_like(ctx.saved_tensors[3])
+        else:
+            saved = ctx.saved_tensors
+            last, sort_status = saved[11], saved[12]
+            last_depth = saved[13] if ctx.has_last_depth else None
+            width, height, tile_width, tile_height, threshold, per_pixel_sort, max_layers = ctx.render_args
+            if grad_image is None:
+                grad_image = torch.zeros_like(saved[7])
+            if grad_depthmap is None:
+                grad_depthmap = torch.zeros_like(saved[8])
+            grad_vertices, grad_colors, grad_opacities = _C.render_backward(
+                grad_image, grad_depthmap, *saved[:11], width, height, tile_width, tile_height, threshold, per_pixel_sort,
+                max_layers, resume=(last, last_depth, sort_status))
+        # one slot per forward argument (wrapper.py:99-112)
+        return (grad_vertices, None, grad_colors, grad_opacities, None, None, None, None, None, None, None, None)
+
+
+def render(
+    vertices: torch.Tensor,
+    indices: torch.Tensor,
+    colors: torch.Tensor,
+    opacities: torch.Tensor,
+    width: int = 500,
+    height: int = 500,
+    tile_width: int = 16,
+    tile_height: int = 16,
+    early_stopping_threshold: float = 1 / 256,
+    record_timing: bool = False,
+    per_pixel_sort: bool = True,
+    max_layers: int = 32,
+) -> Tuple[torch.Tensor, ...]:
+    """
+    Render semi-transparent triangles with the tile rasterizer.
+        vertices : (N, 4) vertices (x'/w', y'/w', z'/w', 1/w') in [-1,1] clip space
+        indices : (M, 3) int32 vertex indices of the triangles
+        colors : (N, 3) vertex colours
+        opacities : (N,) vertex opacities
+        per_pixel_sort : order fragments per pixel (True) or per tile (False)
+        max_layers : maximum number of fragments composited per pixel, <= 0 for no limit
+
+    Returns:
+        image : (height, width, 4); channel 3 holds the remaining transmittance, not opacity
+        depthmap : (height, width)
+        timings (only if record_timing) : dict of seconds per stage
+    """
+    if tile_width * tile_height > 1024:
+        raise ValueError("tile_width * tile_height must be <= 1024")
+    return Renderer.apply(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                          early_stopping_threshold, record_timing, per_pixel_sort, max_layers)
