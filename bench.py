@@ -1,0 +1,187 @@
+#!/usr/bin/env python3
+"""Benchmark of the differentiable tile rasterizer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--mode B]
+
+A step is one forward + backward pass of `trigrad_amd.render` (L2 loss against a
+seeded random target) over one synthetic frame that is already resident in HBM.
+The default workload is configuration 2 of BASELINE.json (1,000,000 triangles,
+1920x1080, float32, 16x16 tiles).  One JSON line is printed:
+
+  value            forward+backward frames/s (the headline metric)
+  roofline         the dominant HBM-bound kernel (one radix-sort sweep pass):
+                   algorithmic bytes per launch / average launch duration from
+                   events recorded on the launch stream, against 8 TB/s
+  cpu_baseline     the CPU oracle (oracle/, a restatement of the reference's
+                   algorithm; the reference has no CPU path) on the same frame,
+                   OpenMP over tiles on the host cores of this box
+  extra            forward-only frames/s, the other compositing mode, sort
+                   Gkeys/s in-frame and on 10^7 synthetic keys, per-stage times,
+                   binning+sort+ranges fraction of the HBM roofline
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+MODES = {
+    "A": dict(per_pixel_sort=True, max_layers=32),    # API defaults
+    "B": dict(per_pixel_sort=False, max_layers=-1),   # tile-order compositing, early termination, full reverse traversal
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--mode", choices=sorted(MODES), default="B")
+    ap.add_argument("--sort-keys", type=int, default=10_000_000)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import trigrad_amd
+    from trigrad_amd import _C, scenes
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    scene = scenes.config(args.config)
+    W, H = scene["width"], scene["height"]
+    M = scene["indices"].shape[0]
+    T = _C.num_tiles(W, H, 16, 16)
+    d = {k: torch.from_numpy(v).to(dev) for k, v in scene.items() if isinstance(v, np.ndarray)}
+    verts = d["vertices"].clone().requires_grad_()
+    colors = d["colors"].clone().requires_grad_()
+    opac = d["opacities"].clone().requires_grad_()
+
+    def step(mode, backward=True):
+        verts.grad = colors.grad = opac.grad = None
+        image, depthmap = trigrad_amd.render(verts, d["indices"], colors, opac, W, H, 16, 16, 1 / 256, False, **MODES[mode])
+        if backward:
+            loss = ((image - d["target"]) ** 2).mean()
+            loss.backward()
+        return image
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1000.0 / steps
+
+    ms = timed(lambda: step(args.mode), args.steps, args.warmup)
+
+    # ---- per-kernel durations from events on the launch stream -------------------
+    _C.profile_enable(True)
+    _C.profile_report()
+    prof_steps = max(3, min(args.steps, 10))
+    for _ in range(prof_steps):
+        step(args.mode)
+    torch.cuda.synchronize()
+    prof = _C.profile_report()
+    _C.profile_enable(False)
+    counts = _C.bin_count(d["vertices"], d["indices"], W, H, 16, 16)
+    K = int(counts.sum().item())
+    passes = (_C.key_bits(T) + 7) // 8
+    sweep_n, sweep_ms = prof["sort_sweep_kernel"]
+    sweep_avg_s = sweep_ms / sweep_n / 1000.0
+    sweep_bytes = 24.0 * K
+    achieved = sweep_bytes / sweep_avg_s / 1e9
+    per_step = {k: v[1] / prof_steps for k, v in prof.items()}
+    bin_sort_kernels = ["bin_count_kernel", "scan_init_kernel", "scan_lookback_kernel", "bin_emit_kernel", "fill_zero_kernel",
+                        "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel", "tile_ranges_kernel"]
+    bin_sort_ms = sum(per_step.get(k, 0.0) for k in bin_sort_kernels)
+    bin_sort_bytes = 136.0 * M + 28.0 * K + 24.0 * passes * K + 4.0 * (T + 1)
+    sort_ms = sum(per_step.get(k, 0.0) for k in ("fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel"))
+
+    out = {
+        "metric": "fwd+bwd frames/s (1M tris, 1920x1080)" if args.config == 2 else f"fwd+bwd frames/s (config {args.config})",
+        "value": 1000.0 / ms,
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"config{args.config}: {M} triangles, {W}x{H}, 16x16 tiles, K={K} keys, "
+                               f"per_pixel_sort={MODES[args.mode]['per_pixel_sort']}, max_layers={MODES[args.mode]['max_layers']}",
+                   "mode": args.mode},
+        "roofline": {"bound": "hbm", "kernel": "sort_sweep_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_launch": sweep_bytes, "avg_launch_us": sweep_avg_s * 1e6},
+    }
+
+    extra = {
+        "kernel_ms_per_step": {k: round(v, 4) for k, v in sorted(per_step.items())},
+        "binning_sort_ranges": {"ms": bin_sort_ms, "algorithmic_bytes": bin_sort_bytes,
+                                "GBps": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9,
+                                "frac_of_hbm_peak": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS},
+        "sort_in_frame": {"keys": K, "passes": passes, "ms": sort_ms, "Gkeys_per_s": K / (sort_ms / 1000.0) / 1e9},
+    }
+    if not args.no_extras:
+        extra["forward_only_fps"] = 1000.0 / timed(lambda: step(args.mode, backward=False), args.steps, 1)
+        other = "A" if args.mode == "B" else "B"
+        extra[f"mode_{other}_fwd_bwd_fps"] = 1000.0 / timed(lambda: step(other), max(3, args.steps // 2), 1)
+        extra[f"mode_{other}_forward_only_fps"] = 1000.0 / timed(lambda: step(other, backward=False), max(3, args.steps // 2), 1)
+        # standalone sort at the scale the metric names
+        n = args.sort_keys
+        keys_np, vals_np = scenes.sort_keys(n, T, seed=0)
+        keys0 = torch.from_numpy(keys_np.view(np.int64)).to(dev)
+        vals0 = torch.from_numpy(vals_np).to(dev)
+        kbuf, vbuf = torch.empty_like(keys0), torch.empty_like(vals0)
+
+        def sort_once():
+            kbuf.copy_(keys0)
+            vbuf.copy_(vals0)
+            _C.sort_pairs(kbuf, vbuf, _C.key_bits(T))
+
+        def copy_only():
+            kbuf.copy_(keys0)
+            vbuf.copy_(vals0)
+        t_sort = timed(sort_once, 10, 2) - timed(copy_only, 10, 2)
+        extra["sort_standalone"] = {"keys": n, "ms": t_sort, "Gkeys_per_s": n / (t_sort / 1000.0) / 1e9,
+                                    "GBps": (8.0 + 24.0 * passes) * n / (t_sort / 1000.0) / 1e9}
+    out["extra"] = extra
+
+    if not args.no_cpu_baseline:
+        from oracle import oracle as O
+        cores = min(O.max_threads(), len(os.sched_getaffinity(0)), 16)
+        O.set_threads(cores)
+        m = MODES[args.mode]
+        v, i, c, o = scene["vertices"], scene["indices"], scene["colors"], scene["opacities"]
+        t0 = time.perf_counter()
+        fwd = O.render(v, i, c, o, W, H, 16, 16, 1 / 256, m["per_pixel_sort"], m["max_layers"])
+        t1 = time.perf_counter()
+        gi = (2.0 * (fwd["image"] - scene["target"]) / fwd["image"].size).astype(np.float32)
+        O.render_backward(gi, np.zeros((H, W), np.float32), v, i, c, o, fwd, W, H, 16, 16, m["per_pixel_sort"], m["max_layers"])
+        t2 = time.perf_counter()
+        out["cpu_baseline"] = {"value": 1.0 / (t2 - t0), "unit": "frames/s", "cores": cores, "kind": "port",
+                               "sample": f"one full forward+backward frame of the same workload (forward {t1 - t0:.2f} s, "
+                                         f"backward {t2 - t1:.2f} s), binning serial, sort/blend/backward OpenMP over tiles"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -44,6 +44,15 @@ const char *tg_last_error(void);
 /* Number of tiles of a W x H image (reference render.cu:105-106). */
 int tg_num_tiles(int width, int height, int tile_w, int tile_h);
 
+/* Per-kernel timing, the counterpart of the reference's CudaTimer
+ * (render.cu:11-49).  While enabled, every kernel launch of the library is
+ * bracketed by events on its stream.  tg_profile_report waits for them, writes
+ * one line "kernel_name launches total_milliseconds" per kernel into buffer
+ * (host, NUL-terminated, truncated to capacity), forgets them, and returns the
+ * length of the full text. */
+void tg_profile_enable(int on);
+int tg_profile_report(char *buffer, size_t capacity);
+
 /* ---- (1) tile binning ------------------------------------------------------- */
 
 /* Per-triangle screen bounds and tile-overlap count: tri_counts[i] = number of

@@ -252,3 +252,21 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
             _ptr(grad_opacities), _stream(vertices)), "tg_render_backward")
     return grad_vertices, grad_colors, grad_opacities
+
+
+# ---- per-kernel timing (the library's counterpart of the reference's CudaTimer) ----
+
+def profile_enable(on=True):
+    _lib.load().tg_profile_enable(1 if on else 0)
+
+
+def profile_report():
+    """-> {kernel_name: (launches, total_milliseconds)} since the last report; waits for the recorded events."""
+    lib = _lib.load()
+    buf = C.create_string_buffer(1 << 16)
+    lib.tg_profile_report(buf, len(buf))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, ms = line.split()
+        out[name] = (int(count), float(ms))
+    return out

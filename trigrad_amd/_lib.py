@@ -21,6 +21,8 @@ SIGNATURES = {
     "tg_version": (_i, []),
     "tg_last_error": (C.c_char_p, []),
     "tg_num_tiles": (_i, [_i, _i, _i, _i]),
+    "tg_profile_enable": (None, [_i]),
+    "tg_profile_report": (_i, [C.c_char_p, _sz]),
     "tg_bin_count": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _p]),
     "tg_scan_workspace_bytes": (_sz, [_i64]),
     "tg_scan_exclusive_u32": (_i, [_p, _p, _i64, _p, _p, _sz, _p, _p]),

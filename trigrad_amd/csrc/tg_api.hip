@@ -1,6 +1,11 @@
-// tg_api.hip -- version, error reporting and helpers shared by every entry point.
+// tg_api.hip -- version, error reporting, per-kernel timing; helpers shared by every entry point.
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
 
 #include "tg_common.hpp"
 
@@ -24,6 +29,33 @@ int check_launch(const char *what) {
     return 0;
 }
 
+// ---- per-kernel timing ---------------------------------------------------------
+struct ProfileRecord {
+    const char *name;
+    hipEvent_t start, stop;
+};
+static bool g_profile_on = false;
+static std::mutex g_profile_mutex;
+static std::vector<ProfileRecord> g_profile_records;
+
+ProfileScope::ProfileScope(const char *name, hipStream_t s) : slot(-1), stream(s) {
+    if (!g_profile_on) return;
+    ProfileRecord r;
+    r.name = name;
+    if (hipEventCreate(&r.start) != hipSuccess) return;
+    if (hipEventCreate(&r.stop) != hipSuccess) { (void)hipEventDestroy(r.start); return; }
+    (void)hipEventRecord(r.start, s);
+    std::lock_guard<std::mutex> lock(g_profile_mutex);
+    slot = (int)g_profile_records.size();
+    g_profile_records.push_back(r);
+}
+
+ProfileScope::~ProfileScope() {
+    if (slot < 0) return;
+    std::lock_guard<std::mutex> lock(g_profile_mutex);
+    if (slot < (int)g_profile_records.size()) (void)hipEventRecord(g_profile_records[slot].stop, stream);
+}
+
 }  // namespace tg
 
 extern "C" int tg_version(void) { return TG_ABI_VERSION; }
@@ -33,4 +65,38 @@ extern "C" const char *tg_last_error(void) { return tg::g_error; }
 extern "C" int tg_num_tiles(int width, int height, int tile_w, int tile_h) {
     if (width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0) return 0;
     return tg::ceil_div(width, tile_w) * tg::ceil_div(height, tile_h);
+}
+
+extern "C" void tg_profile_enable(int on) { tg::g_profile_on = on != 0; }
+
+extern "C" int tg_profile_report(char *buffer, size_t capacity) {
+    using namespace tg;
+    std::vector<ProfileRecord> records;
+    {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
+        records.swap(g_profile_records);
+    }
+    struct Sum { long count = 0; double ms = 0.0; };
+    std::map<std::string, Sum> sums;
+    for (const ProfileRecord &r : records) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+            Sum &s = sums[r.name];
+            s.count++;
+            s.ms += ms;
+        }
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    std::string text;
+    char line[256];
+    for (const auto &kv : sums) {
+        snprintf(line, sizeof(line), "%s %ld %.6f\n", kv.first.c_str(), kv.second.count, kv.second.ms);
+        text += line;
+    }
+    if (!buffer || capacity == 0) return (int)text.size();
+    const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+    memcpy(buffer, text.data(), n);
+    buffer[n] = '\0';
+    return (int)text.size();
 }

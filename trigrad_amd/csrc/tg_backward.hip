@@ -429,13 +429,13 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
-        hipLaunchKernelGGL(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
+        TG_LAUNCH(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
         return check_launch("backward_tile_order_kernel");
     }
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads());
     const size_t lds = pixel_order_lds_bytes(tl.threads);
     static size_t lds_reserved = 0;
     if (int e = reserve_lds("tg_render_backward", (const void *)backward_pixel_order_kernel, lds, &lds_reserved)) return e;
-    hipLaunchKernelGGL(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds, s, a, g);
+    TG_LAUNCH(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds, s, a, g);
     return check_launch("backward_pixel_order_kernel");
 }

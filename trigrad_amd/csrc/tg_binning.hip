@@ -197,7 +197,7 @@ extern "C" int tg_bin_count(const float *vertices, int32_t n_vertices, const int
     if (int e = check_geometry("tg_bin_count", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
     if (n_triangles == 0) return 0;
     if (!tri_counts) { set_error("tg_bin_count: tri_counts is null"); return TG_E_ARG; }
-    hipLaunchKernelGGL(bin_count_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+    TG_LAUNCH(bin_count_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
                        (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
                        ceil_div(width, tile_w), ceil_div(height, tile_h), tri_counts);
     return check_launch("bin_count_kernel");
@@ -210,7 +210,7 @@ extern "C" int tg_bin_emit(const float *vertices, int32_t n_vertices, const int3
     if (n_keys < 0 || n_keys > 0xffffffffll) { set_error("tg_bin_emit: n_keys out of range"); return TG_E_ARG; }
     if (n_keys == 0) return 0;
     if (n_triangles == 0 || !tri_offsets || !keys || !payload) { set_error("tg_bin_emit: null pointer"); return TG_E_ARG; }
-    hipLaunchKernelGGL(bin_emit_kernel, dim3((unsigned)ceil_div64(n_keys, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+    TG_LAUNCH(bin_emit_kernel, dim3((unsigned)ceil_div64(n_keys, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
                        (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
                        ceil_div(width, tile_w), ceil_div(height, tile_h), tri_offsets, n_keys, keys, payload);
     return check_launch("bin_emit_kernel");
@@ -221,7 +221,7 @@ extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n
         set_error("tg_tile_ranges: null pointer or size out of range");
         return TG_E_ARG;
     }
-    hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)ceil_div64(n_keys + 1, kBinThreads)), dim3(kBinThreads), 0,
+    TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n_keys + 1, kBinThreads)), dim3(kBinThreads), 0,
                        (hipStream_t)stream, sorted_keys, n_keys, n_tiles, offsets);
     return check_launch("tile_ranges_kernel");
 }
@@ -231,7 +231,7 @@ extern "C" int tg_bary(const float *vertices, int32_t n_vertices, const int32_t 
     if (int e = check_geometry("tg_bary", vertices, n_vertices, indices, n_triangles, 1, 1, 1, 1)) return e;
     if (n_triangles == 0) return 0;
     if (!out) { set_error("tg_bary: out is null"); return TG_E_ARG; }
-    hipLaunchKernelGGL(bary_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+    TG_LAUNCH(bary_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
                        (const float4 *)vertices, n_vertices, indices, n_triangles, out);
     return check_launch("bary_kernel");
 }

@@ -24,6 +24,22 @@ constexpr int kWave = 64;
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
 
+// Per-kernel timing (the counterpart of the reference's CudaTimer,
+// render.cu:11-49): when enabled through tg_profile_enable, every launch is
+// bracketed by a pair of events on its stream; tg_profile_report waits for
+// them and sums the elapsed time per kernel name.
+struct ProfileScope {
+    ProfileScope(const char *name, hipStream_t stream);
+    ~ProfileScope();
+    int slot;
+    hipStream_t stream;
+};
+#define TG_LAUNCH(kernel, grid, block, lds, stream, ...)               \
+    do {                                                               \
+        tg::ProfileScope tg_profile_scope(#kernel, stream);            \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__); \
+    } while (0)
+
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -234,12 +234,12 @@ extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, 
     const int n_threads = tl.threads;
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {
-        hipLaunchKernelGGL(forward_tile_order_kernel, grid, dim3(n_threads), 0, s, a, o);
+        TG_LAUNCH(forward_tile_order_kernel, grid, dim3(n_threads), 0, s, a, o);
         return check_launch("forward_tile_order_kernel");
     }
     const size_t lds = pixel_order_lds_bytes(n_threads);
     static size_t lds_reserved = 0;
     if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel, lds, &lds_reserved)) return e;
-    hipLaunchKernelGGL(forward_pixel_order_kernel, grid, dim3(n_threads), lds, s, a, o);
+    TG_LAUNCH(forward_pixel_order_kernel, grid, dim3(n_threads), lds, s, a, o);
     return check_launch("forward_pixel_order_kernel");
 }

@@ -173,10 +173,10 @@ extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t 
     uint32_t *ticket = (uint32_t *)workspace;
     uint64_t *states = (uint64_t *)((char *)workspace + scan_state_offset());
     const int init_blocks = n_tiles > 0 ? ceil_div(n_tiles, 256) : 1;
-    hipLaunchKernelGGL(scan_init_kernel, dim3(init_blocks), dim3(256), 0, s, ticket, states, n_tiles, total, status);
+    TG_LAUNCH(scan_init_kernel, dim3(init_blocks), dim3(256), 0, s, ticket, states, n_tiles, total, status);
     if (int e = check_launch("scan_init_kernel")) return e;
     if (n_tiles == 0) return 0;
-    hipLaunchKernelGGL(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
+    TG_LAUNCH(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
                        n_tiles, status);
     return check_launch("scan_lookback_kernel");
 }

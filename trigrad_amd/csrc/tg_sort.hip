@@ -262,7 +262,7 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
     *result_in_alt = 0;
     hipStream_t s = (hipStream_t)stream;
     if (status) {
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
+        TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
         if (int e = check_launch("fill_zero_kernel")) return e;
     }
     if (n == 0 || end_bit == 0) return 0;
@@ -286,22 +286,22 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
     uint32_t *lookback = (uint32_t *)(ws + L.off_lookback);
 
     // tickets and look-back words start at zero; bases and partials are fully overwritten
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, tickets, (size_t)64);
+    TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, tickets, (size_t)64);
     if (int e = check_launch("fill_zero_kernel")) return e;
     const size_t lb_words = (size_t)L.passes * L.n_tiles * kRadix;
     const int fill_blocks = (int)((lb_words + 1023) / 1024 < 2048 ? (lb_words + 1023) / 1024 : 2048);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, lookback, lb_words);
+    TG_LAUNCH(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, lookback, lb_words);
     if (int e = check_launch("fill_zero_kernel")) return e;
 
-    hipLaunchKernelGGL(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials);
+    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials);
     if (int e = check_launch("sort_histogram_kernel")) return e;
-    hipLaunchKernelGGL(sort_bases_kernel, dim3(L.passes), dim3(kSortThreads), 0, s, partials, L.hist_blocks, bases);
+    TG_LAUNCH(sort_bases_kernel, dim3(L.passes), dim3(kSortThreads), 0, s, partials, L.hist_blocks, bases);
     if (int e = check_launch("sort_bases_kernel")) return e;
 
     uint64_t *kin = keys, *kout = keys_alt;
     uint32_t *vin = values, *vout = values_alt;
     for (int p = 0; p < L.passes; p++) {
-        hipLaunchKernelGGL(sort_sweep_kernel, dim3(L.n_tiles), dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, p * kRadixBits,
+        TG_LAUNCH(sort_sweep_kernel, dim3(L.n_tiles), dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, p * kRadixBits,
                            bases + p * kRadix, lookback + (size_t)p * L.n_tiles * kRadix, tickets + p, status);
         if (int e = check_launch("sort_sweep_kernel")) return e;
         uint64_t *tk = kin; kin = kout; kout = tk;
