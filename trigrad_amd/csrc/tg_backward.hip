@@ -91,13 +91,22 @@ __device__ __forceinline__ void interp_backward_scalar(float g, const float b[3]
     }
 }
 
-// The arithmetic of process_backward (render.cu:455-538) for a fragment known
-// to be inside; `out` receives the 21 gradient terms.
-__device__ __forceinline__ void fragment_backward(BackState &st, const BackRecord &r, float b0, float b1, float b2, float px,
-                                                  float py, float out[kTerms]) {
-    const float b[3] = {b0, b1, b2};
+// process_backward (render.cu:455-538) is evaluated in two parts.  The part that
+// carries state from one fragment of a pixel to the next (transmittance and the
+// running sums) has to follow the reverse blend order of that pixel; it reduces
+// the fragment to five numbers.  Everything else is a function of those five
+// numbers, the pixel position and the triangle, and can be evaluated in any
+// order.
+
+// What the ordered part hands over for one fragment.
+struct FragSeed {
+    float d_do;    // derivative w.r.t. the interpolated opacity (:502)
+    float gc[3];   // derivative w.r.t. the interpolated colour (:510)
+    float dd_dz;   // derivative w.r.t. the interpolated view depth (:517)
+};
+
+__device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, float b0, float b1, float b2) {
     const float w[3] = {r.w[0], r.w[1], r.w[2]};
-    const float ones[3] = {1.0f, 1.0f, 1.0f};
     float o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
     o = clampf(o, 0.0f, kMaxOpacity);
     float color[3];
@@ -122,14 +131,26 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
     st.zoa = st.zoa + z * o * st.alpha;                                                // :497
     float dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
     if (st.final_weight < kEffZero) dd_do = 0.0f;
-    const float d_do = drgb_do + dd_do;
+    FragSeed f;
+    f.d_do = drgb_do + dd_do;
+    const float ao = st.alpha * o;
+    f.gc[0] = ao * g[0]; f.gc[1] = ao * g[1]; f.gc[2] = ao * g[2];                     // :510
+    f.dd_dz = ao * st.gd / st.final_weight;                                            // :517
+    if (st.final_weight < kEffZero) f.dd_dz = 0.0f;
+    return f;
+}
 
+// The order-free part: the 21 gradient terms of one fragment.
+__device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackRecord &r, float b0, float b1, float b2, float px,
+                                               float py, float out[kTerms]) {
+    const float b[3] = {b0, b1, b2};
+    const float w[3] = {r.w[0], r.w[1], r.w[2]};
+    const float ones[3] = {1.0f, 1.0f, 1.0f};
     float gb_o[3], gv_o[3], gw_o[3];
-    interp_backward_scalar(d_do, b, r.op, w, gb_o, gv_o, gw_o);
+    interp_backward_scalar(f.d_do, b, r.op, w, gb_o, gv_o, gw_o);
 
     // vector interpolate3_backward for the colour (util.h:319-355)
-    const float ao = st.alpha * o;
-    const float gc[3] = {ao * g[0], ao * g[1], ao * g[2]};  // :510
+    const float *gc = f.gc;
     float gb_c[3] = {0.f, 0.f, 0.f}, gw_c[3] = {0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f};
     {
         float nom[3];
@@ -154,10 +175,8 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
         }
     }
 
-    float dd_dz = ao * st.gd / st.final_weight;  // :517
-    if (st.final_weight < kEffZero) dd_dz = 0.0f;
     float gb_z[3], gv_z[3], gw_z[3];
-    interp_backward_scalar(dd_dz, b, r.iw, ones, gb_z, gv_z, gw_z);
+    interp_backward_scalar(f.dd_dz, b, r.iw, ones, gb_z, gv_z, gw_z);
 
     float gbary[3];
 #pragma unroll
@@ -212,6 +231,13 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
     }
 }
 
+// One fragment start to finish (used where every pixel has its own order).
+__device__ __forceinline__ void fragment_backward(BackState &st, const BackRecord &r, float b0, float b1, float b2, float px,
+                                                  float py, float out[kTerms]) {
+    const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
+    fragment_terms(f, r, b0, b1, b2, px, py, out);
+}
+
 __device__ __forceinline__ float *term_address(const BackwardArgs &g, int vertex_id, int c) {
     if (c < 2) return g.grad_vertices + 4 * (int64_t)vertex_id + c;
     if (c == 2) return g.grad_vertices + 4 * (int64_t)vertex_id + 3;
@@ -233,32 +259,68 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
     return st;
 }
 
-// Sum over the 64 lanes of a wave, result valid in lane 63.
-__device__ __forceinline__ float wave_reduce_add(float v) {
-#define TG_DPP_ADD(ctrl, rows) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rows, 0xf, false))
-    TG_DPP_ADD(0x111, 0xf);  // row_shr:1
-    TG_DPP_ADD(0x112, 0xf);  // row_shr:2
-    TG_DPP_ADD(0x114, 0xf);  // row_shr:4
-    TG_DPP_ADD(0x118, 0xf);  // row_shr:8
-    TG_DPP_ADD(0x142, 0xa);  // row_bcast:15
-    TG_DPP_ADD(0x143, 0xc);  // row_bcast:31
-#undef TG_DPP_ADD
-    return v;
+constexpr int kBackBatch = 128;   // list entries staged per batch
+constexpr int kWaveSlots = 256;   // hit slots per wave and round
+constexpr int kSeedWords = 6;     // d_do, gc[3], dd_dz, (entry | source lane << 8)
+constexpr int kTermStride = 65;   // row stride of the per-wave term matrix (odd: conflict-free columns)
+constexpr int kMaxWaves = kTileThreads / kWave;
+
+__device__ __forceinline__ int top_bit(uint64_t m) { return 63 - __builtin_clzll(m); }
+
+__device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
-constexpr int kDenseHits = 12;  // lanes of a wave hitting one entry from which the DPP reduction pays
+// Orders the LDS traffic of one wave: what lanes wrote before is visible to the
+// lanes that read after (LDS serves a wave's instructions in order; this keeps
+// the compiler from moving accesses across the point).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
+// Tile-order backward.  LDS float atomics cost about three cycles per lane on
+// gfx950 and direct global atomics collide on the shared vertices, so the
+// per-entry sums are formed with plain LDS stores and loads.  The records of
+// 128 list entries are staged per batch by the whole workgroup; after that
+// every wave works on its own 64 pixels without workgroup barriers:
+//   1. every lane tests its pixel against every record (same record for all
+//      lanes: LDS broadcast) and keeps its hits as a 128-bit mask; the wave's
+//      ballot per record is stored;
+//   2. the ballots become slot numbers: entries from the far end, lanes in
+//      order inside an entry, so every (pixel, entry) hit of the wave owns one
+//      slot, slots are grouped by entry, and a lane's own hits have increasing
+//      numbers in the order it must visit them (reverse blend order);
+//   3. ordered part, in rounds of 256 slots: every lane walks its own hits and
+//      advances the pixel's transmittance and running sums; each hit leaves
+//      five numbers in its slot;
+//   4. order-free part, 64 slots at a time with every lane busy: lane = slot
+//      evaluates the 21 gradient terms of its hit and writes them to a term
+//      matrix; three groups of 21 lanes add up the runs of equal entry and issue
+//      one global float atomic per run and term.
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
-    __shared__ BackRecord s_rec[kBatch];
-    __shared__ float s_acc[kBatch * kTerms];
+    __shared__ BackRecord s_rec[kBackBatch];
+    __shared__ uint64_t s_ballot[kMaxWaves][kBackBatch];
+    __shared__ uint32_t s_base[kMaxWaves][kBackBatch];
+    __shared__ float s_seed[kMaxWaves][kSeedWords][kWaveSlots];
+    __shared__ float s_term[kMaxWaves][kTerms * kTermStride];
+    __shared__ float s_px[kTileThreads], s_py[kTileThreads];
     __shared__ int s_last;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile];
     const PixelCoord p = pixel_of_thread(a);
+    uint64_t *ballots = s_ballot[wave];
+    uint32_t *bases = s_base[wave];
+    float (*seeds)[kWaveSlots] = s_seed[wave];
+    float *terms = s_term[wave];
 
     if (tid == 0) s_last = 0;
+    s_px[tid] = p.px;
+    s_py[tid] = p.py;
     __syncthreads();
     const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
     if (my_last > 0) atomicMax(&s_last, my_last);
@@ -268,45 +330,123 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     BackState st;
     if (p.valid) st = load_back_state(g, p);
 
-    for (int hi = tile_last; hi > 0; hi -= kBatch) {
-        const int lo = max(0, hi - kBatch);
+    for (int hi = tile_last; hi > 0; hi -= kBackBatch) {
+        const int lo = max(0, hi - kBackBatch);
         const int nb = hi - lo;
-        __syncthreads();  // the previous batch's flush has finished
+        __syncthreads();  // every wave is done with the previous batch
         for (int e = tid; e < nb; e += blockDim.x) gather_back(a, start + lo + e, s_rec[e]);
-        for (int i = tid; i < nb * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
         __syncthreads();
-        for (int e = nb - 1; e >= 0; e--) {
-            const BackRecord &r = s_rec[e];
-            bool hit = false;
-            float b0 = 0.f, b1 = 0.f, b2 = 0.f;
-            if (lo + e < my_last) {
+
+        // 1. inside tests
+        const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
+        if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
+        uint64_t m[2] = {0, 0};
+#pragma unroll
+        for (int wd = 0; wd < 2; wd++) {
+            uint64_t bits = 0;
+            const int count = min(64, nb - 64 * wd);
+            for (int bit = 0; bit < count; bit++) {
+                const BackRecord &r = s_rec[64 * wd + bit];
+                float b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                hit = bary_inside(b0, b1, b2);
+                const bool hit = bary_inside(b0, b1, b2) && 64 * wd + bit < mine;
+                const uint64_t vote = __builtin_amdgcn_ballot_w64(hit);
+                if (hit) bits |= 1ull << bit;
+                if (lane == 0) ballots[64 * wd + bit] = vote;
             }
-            const uint64_t hits = __builtin_amdgcn_ballot_w64(hit);
-            if (hits == 0) continue;  // wave-uniform
-            float term[kTerms];
-#pragma unroll
-            for (int q = 0; q < kTerms; q++) term[q] = 0.0f;
-            if (hit) fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
-            float *acc = s_acc + e * kTerms;
-            if (__builtin_popcountll(hits) >= kDenseHits) {
-#pragma unroll
-                for (int q = 0; q < kTerms; q++) {
-                    const float sum = wave_reduce_add(term[q]);
-                    if (lane == kWave - 1) atomicAdd(acc + q, sum);
-                }
-            } else if (hit) {
-#pragma unroll
-                for (int q = 0; q < kTerms; q++) atomicAdd(acc + q, term[q]);
-            }
+            m[wd] = bits;
         }
-        __syncthreads();
-        for (int i = tid; i < nb * kTerms; i += blockDim.x) {
-            const float v = s_acc[i];
-            if (v != 0.0f) {
-                const int e = i / kTerms, q = i - e * kTerms;
-                unsafeAtomicAdd(term_address(g, s_rec[e].id[q / 7], q % 7), v);
+        wave_lds_sync();
+
+        // 2. slot numbers of this wave
+        uint32_t n_hits;
+        {
+            uint32_t cnt[2];
+            const int e0 = nb - 1 - 2 * lane, e1 = e0 - 1;
+            cnt[0] = e0 >= 0 ? (uint32_t)__builtin_popcountll(ballots[e0]) : 0u;
+            cnt[1] = e1 >= 0 ? (uint32_t)__builtin_popcountll(ballots[e1]) : 0u;
+            const uint32_t incl = wave_inclusive_scan_u32(cnt[0] + cnt[1]);
+            const uint32_t excl = incl - cnt[0] - cnt[1];
+            if (e0 >= 0) bases[e0] = excl;
+            if (e1 >= 0) bases[e1] = excl + cnt[0];
+            n_hits = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        }
+        wave_lds_sync();
+
+        for (uint32_t round0 = 0; round0 < n_hits; round0 += kWaveSlots) {
+            // 3. ordered part, lane by lane over its own hits
+            while (true) {
+                int e = -1;
+                uint32_t slot = 0;
+                if (m[1]) e = 64 + top_bit(m[1]);
+                else if (m[0]) e = top_bit(m[0]);
+                if (e >= 0) {
+                    slot = bases[e] + lanes_below_mask(ballots[e]) - round0;
+                    if (slot >= (uint32_t)kWaveSlots) e = -1;  // this hit, and all my later ones, belong to a later round
+                }
+                const bool active = e >= 0;
+                if (__builtin_amdgcn_ballot_w64(active) == 0) break;  // wave-uniform
+                if (active) {
+                    if (e >= 64) m[1] &= ~(1ull << (e - 64)); else m[0] &= ~(1ull << e);
+                    const BackRecord &r = s_rec[e];
+                    float b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
+                    seeds[0][slot] = f.d_do;
+                    seeds[1][slot] = f.gc[0];
+                    seeds[2][slot] = f.gc[1];
+                    seeds[3][slot] = f.gc[2];
+                    seeds[4][slot] = f.dd_dz;
+                    seeds[5][slot] = __int_as_float(e | (lane << 8));
+                }
+            }
+            wave_lds_sync();
+
+            // 4. order-free part
+            const int n_slots = (int)min((uint32_t)kWaveSlots, n_hits - round0);
+            for (int s0 = 0; s0 < n_slots; s0 += kWave) {
+                const int n_here = min(kWave, n_slots - s0);
+                int tag = -1;
+                if (lane < n_here) {
+                    const int slot = s0 + lane;
+                    FragSeed f;
+                    f.d_do = seeds[0][slot];
+                    f.gc[0] = seeds[1][slot];
+                    f.gc[1] = seeds[2][slot];
+                    f.gc[2] = seeds[3][slot];
+                    f.dd_dz = seeds[4][slot];
+                    const int packed = __float_as_int(seeds[5][slot]);
+                    tag = packed & 0xff;
+                    const int src = wave * kWave + (packed >> 8);
+                    const float px = s_px[src], py = s_py[src];
+                    const BackRecord &r = s_rec[tag];
+                    float b0, b1, b2;
+                    bary_apply(r.m, px, py, b0, b1, b2);
+                    float term[kTerms];
+                    fragment_terms(f, r, b0, b1, b2, px, py, term);
+#pragma unroll
+                    for (int q = 0; q < kTerms; q++) terms[q * kTermStride + lane] = term[q];
+                }
+                wave_lds_sync();
+                // lanes (group, q): group 0..2 owns a third of the slots; runs of equal entry are contiguous
+                const int group = lane / kTerms, q = lane - group * kTerms;
+                const int per = (n_here + 2) / 3;
+                const int c0 = group * per, c1 = min(c0 + per, n_here);
+                if (group < 3 && c0 < c1) {
+                    int cur = __float_as_int(seeds[5][s0 + c0]) & 0xff;
+                    float acc = 0.0f;
+                    for (int c = c0; c < c1; c++) {
+                        const int t = __float_as_int(seeds[5][s0 + c]) & 0xff;
+                        if (t != cur) {
+                            if (acc != 0.0f) unsafeAtomicAdd(term_address(g, s_rec[cur].id[q / 7], q % 7), acc);
+                            acc = 0.0f;
+                            cur = t;
+                        }
+                        acc += terms[q * kTermStride + c];
+                    }
+                    if (acc != 0.0f) unsafeAtomicAdd(term_address(g, s_rec[cur].id[q / 7], q % 7), acc);
+                }
+                wave_lds_sync();
             }
         }
     }

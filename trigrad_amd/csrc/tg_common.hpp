@@ -119,4 +119,21 @@ __device__ __forceinline__ float pixel_ndc(int i, int extent) {
     return (float)(((double)(float)i + 0.5) / (double)(float)extent * 2.0 - 1.0);
 }
 
+// ---- wave64 DPP scan -----------------------------------------------------------
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ uint32_t dpp_add_u32(uint32_t v) {
+    // lanes whose source is out of range (or whose row is masked off) receive 0
+    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false);
+}
+// Inclusive prefix sum over the 64 lanes of a wave (all lanes must be active).
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
+    v = dpp_add_u32<0x111, 0xf>(v);  // row_shr:1
+    v = dpp_add_u32<0x112, 0xf>(v);  // row_shr:2
+    v = dpp_add_u32<0x114, 0xf>(v);  // row_shr:4
+    v = dpp_add_u32<0x118, 0xf>(v);  // row_shr:8
+    v = dpp_add_u32<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add_u32<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 }  // namespace tg

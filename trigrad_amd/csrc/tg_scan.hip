@@ -24,25 +24,8 @@ constexpr uint32_t kSpinLimit = 1u << 20;
 constexpr uint64_t kFlagAggregate = 1ull << 62;
 constexpr uint64_t kFlagInclusive = 2ull << 62;
 
-template <int kCtrl, int kRowMask>
-__device__ __forceinline__ uint32_t dpp_add(uint32_t v) {
-    // lanes whose source is out of range (or whose row is masked off) receive 0
-    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false);
-}
-
-// Inclusive scan over the 64 lanes of a wave.
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
-    v = dpp_add<0x111, 0xf>(v);  // row_shr:1
-    v = dpp_add<0x112, 0xf>(v);  // row_shr:2
-    v = dpp_add<0x114, 0xf>(v);  // row_shr:4
-    v = dpp_add<0x118, 0xf>(v);  // row_shr:8
-    v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-    v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
 __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
-    v = wave_inclusive_scan(v);
+    v = wave_inclusive_scan_u32(v);
     return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
@@ -80,14 +63,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint3
             if (base + k < n) x[k] = in[base + k];
     }
     const uint32_t thread_sum = x[0] + x[1] + x[2] + x[3];
-    const uint32_t incl = wave_inclusive_scan(thread_sum);
+    const uint32_t incl = wave_inclusive_scan_u32(thread_sum);
     if (lane == kWave - 1) s_wave_total[wave] = incl;
     __syncthreads();
 
     if (wave == 0) {
         // scan of the wave totals, then publish and look back
         uint32_t wt = (lane < kScanThreads / kWave) ? s_wave_total[lane] : 0u;
-        uint32_t wincl = wave_inclusive_scan(wt);
+        uint32_t wincl = wave_inclusive_scan_u32(wt);
         uint32_t tile_total = (uint32_t)__builtin_amdgcn_readlane((int)wincl, kScanThreads / kWave - 1);
         if (lane < kScanThreads / kWave) s_wave_total[lane] = wincl - wt;  // exclusive wave offsets
 
