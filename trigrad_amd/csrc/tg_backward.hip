@@ -452,6 +452,8 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     }
 }
 
+constexpr int kAccWindow = 512;  // list positions whose gradient sums are kept in LDS by the per-pixel-order kernel
+
 // Candidate insertion for the reverse selection: keeps the `cap` LARGEST
 // (depth, position) pairs in descending order.  Positions arrive in ascending
 // order, so a candidate whose depth equals a stored one has the larger position
@@ -477,11 +479,16 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     tk.depth = reinterpret_cast<float *>(s_dyn + sizeof(DepthRecord) * kBatch);
     tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
+    // Per-entry sums of the first kAccWindow list positions live in LDS and are
+    // flushed once per tile; positions beyond the window go straight to memory.
+    float *s_acc = reinterpret_cast<float *>(tk.pos + kLayers * n_threads);
 
     const int tid = threadIdx.x;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
+    const int n_acc = min(end - start, kAccWindow);
+    for (int i = tid; i < n_acc * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
 
     BackState st;
     int remaining = 0;
@@ -525,9 +532,15 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
                 if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
                 float term[kTerms];
                 fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
+                const int rel = tk.j(i) - start;
+                if (rel < kAccWindow) {
 #pragma unroll
-                for (int q = 0; q < kTerms; q++)
-                    if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+                    for (int q = 0; q < kTerms; q++) atomicAdd(s_acc + rel * kTerms + q, term[q]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < kTerms; q++)
+                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+                }
             }
             if (found < cap) {
                 remaining = 0;  // list exhausted
@@ -538,7 +551,19 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
             }
         }
     }
+    __syncthreads();
+    for (int e = tid; e < n_acc; e += blockDim.x) {
+        const TriIds t = load_ids(a, start + e);
+        const int id[3] = {t.ia, t.ib, t.ic};
+#pragma unroll
+        for (int q = 0; q < kTerms; q++) {
+            const float v = s_acc[e * kTerms + q];
+            if (v != 0.0f) unsafeAtomicAdd(term_address(g, id[q / 7], q % 7), v);
+        }
+    }
 }
+
+size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads) + (size_t)kAccWindow * kTerms * sizeof(float); }
 
 }  // namespace tg
 
@@ -573,7 +598,7 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
         return check_launch("backward_tile_order_kernel");
     }
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads());
-    const size_t lds = pixel_order_lds_bytes(tl.threads);
+    const size_t lds = backward_pixel_order_lds_bytes(tl.threads);
     static size_t lds_reserved = 0;
     if (int e = reserve_lds("tg_render_backward", (const void *)backward_pixel_order_kernel, lds, &lds_reserved)) return e;
     TG_LAUNCH(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds, s, a, g);
