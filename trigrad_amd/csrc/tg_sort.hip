@@ -3,11 +3,12 @@
 // HBM-bound: one read of the keys for all digit histograms (8 B/key), then per
 // pass one read and one write of key + value (24 B/key).  Structure:
 //
-//   fill        zero the workspace (tickets, look-back words)
+//   fill        zero the tickets and the look-back words (one launch)
 //   histogram   every workgroup builds the 256-bin histogram of EVERY pass in
 //               LDS (ds_add_u32) from one sweep over the keys and stores it as
 //               a partial (no global atomics)
-//   bases       per pass: sum the partials, exclusive scan over the 256 digits
+//   bases       per pass (one workgroup of 1024 threads): sum the partials,
+//               exclusive scan over the 256 digits
 //   sweep x P   each workgroup owns a tile of 4096 consecutive pairs:
 //                 - wave64 match ranking: 8 ballots find the lanes that hold
 //                   the same digit, mbcnt-style popcounts give the stable rank,
@@ -16,9 +17,10 @@
 //                 - the tile's 256 digit counts are published in look-back
 //                   words (one uint32 per digit: bits 31..30 = 0 not ready,
 //                   1 aggregate, 2 inclusive prefix; bits 29..0 = count) and
-//                   thread d walks back over the predecessors' words of digit d
-//                   (decoupled look-back; relaxed agent-scope atomics suffice as
-//                   flag and value share a word);
+//                   thread d walks back over the predecessors' words of digit d,
+//                   eight words in flight per step (decoupled look-back;
+//                   relaxed agent-scope atomics suffice as flag and value
+//                   share a word);
 //                 - pairs are permuted into digit order through LDS, then each
 //                   digit run is written contiguously.
 //
@@ -35,7 +37,9 @@ constexpr int kSortThreads = 256;
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kSortItems = 16;
 constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
-constexpr int kHistBlocksMax = 512;
+constexpr int kHistBlocksMax = 256;
+constexpr int kBasesThreads = 1024;
+constexpr int kLookWindow = 16;
 constexpr uint32_t kSortSpinLimit = 1u << 20;
 constexpr uint32_t kLbAggregate = 1u << 30;
 constexpr uint32_t kLbInclusive = 2u << 30;
@@ -55,9 +59,9 @@ static SortLayout sort_layout(int64_t n, int end_bit) {
     L.n_tiles = (int)ceil_div64(n, kSortTile);
     L.hist_blocks = L.n_tiles < kHistBlocksMax ? (L.n_tiles > 0 ? L.n_tiles : 1) : kHistBlocksMax;
     size_t o = 0;
-    L.off_tickets = o;  o += 256;  // kMaxPasses tickets, padded
     L.off_bases = o;    o += (size_t)kMaxPasses * kRadix * 4;
     L.off_partials = o; o += (size_t)kHistBlocksMax * kMaxPasses * kRadix * 4;
+    L.off_tickets = o;  o += 256;  // kMaxPasses tickets, padded; zeroed together with the look-back words
     L.off_lookback = o; o += (size_t)kMaxPasses * (size_t)(L.n_tiles > 0 ? L.n_tiles : 1) * kRadix * 4;
     L.total = o;
     return L;
@@ -75,33 +79,50 @@ __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint
     const int tid = threadIdx.x;
     for (int p = 0; p < passes; p++) s_hist[p][tid] = 0;
     __syncthreads();
-    const int64_t stride = (int64_t)gridDim.x * kSortThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kSortThreads + tid; i < n; i += stride) {
-        const uint64_t k = keys[i];
-        for (int p = 0; p < passes; p++) atomicAdd(&s_hist[p][(k >> (p * kRadixBits)) & (kRadix - 1)], 1u);
+    const int64_t stride = (int64_t)gridDim.x * kSortThreads * 4;
+    for (int64_t i = (int64_t)blockIdx.x * kSortThreads * 4 + tid; i < n; i += stride) {
+        uint64_t k[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) k[u] = (i + u * kSortThreads < n) ? keys[i + u * kSortThreads] : 0;
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (i + u * kSortThreads < n)
+                for (int p = 0; p < passes; p++) atomicAdd(&s_hist[p][(k[u] >> (p * kRadixBits)) & (kRadix - 1)], 1u);
     }
     __syncthreads();
     uint32_t *out = partials + (size_t)blockIdx.x * kMaxPasses * kRadix;
     for (int p = 0; p < passes; p++) out[p * kRadix + tid] = s_hist[p][tid];
 }
 
-// One workgroup per pass: digit totals over all partials, then exclusive scan.
-__global__ __launch_bounds__(kSortThreads) void sort_bases_kernel(const uint32_t *__restrict__ partials, int hist_blocks,
-                                                                  uint32_t *__restrict__ bases) {
+// One workgroup per pass: digit totals over all partials (four groups of 256
+// threads share the partials), then exclusive scan over the 256 digits.
+__global__ __launch_bounds__(kBasesThreads) void sort_bases_kernel(const uint32_t *__restrict__ partials, int hist_blocks,
+                                                                   uint32_t *__restrict__ bases, uint32_t *status) {
+    __shared__ uint32_t s_part[kBasesThreads / kRadix][kRadix];
     __shared__ uint32_t s_scan[kRadix];
     const int tid = threadIdx.x;
+    const int digit = tid & (kRadix - 1), group = tid / kRadix;
     const int p = blockIdx.x;
+    if (p == 0 && tid == 0 && status) *status = TG_STATUS_OK;
+    uint32_t sum = 0;
+#pragma unroll 8
+    for (int b = group; b < hist_blocks; b += kBasesThreads / kRadix) sum += partials[((size_t)b * kMaxPasses + p) * kRadix + digit];
+    s_part[group][digit] = sum;
+    __syncthreads();
     uint32_t total = 0;
-    for (int b = 0; b < hist_blocks; b++) total += partials[((size_t)b * kMaxPasses + p) * kRadix + tid];
-    s_scan[tid] = total;
+    if (tid < kRadix) {
+#pragma unroll
+        for (int k = 0; k < kBasesThreads / kRadix; k++) total += s_part[k][tid];
+        s_scan[tid] = total;
+    }
     __syncthreads();
     for (int off = 1; off < kRadix; off <<= 1) {  // Hillis-Steele over 256 entries
-        uint32_t v = (tid >= off) ? s_scan[tid - off] : 0u;
+        uint32_t v = (tid < kRadix && tid >= off) ? s_scan[tid - off] : 0u;
         __syncthreads();
-        s_scan[tid] += v;
+        if (tid < kRadix) s_scan[tid] += v;
         __syncthreads();
     }
-    bases[p * kRadix + tid] = s_scan[tid] - total;
+    if (tid < kRadix) bases[p * kRadix + tid] = s_scan[tid] - total;
 }
 
 __device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
@@ -115,12 +136,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
                                                                   int64_t n, int shift, const uint32_t *__restrict__ bases,
                                                                   uint32_t *lookback, uint32_t *ticket, uint32_t *status) {
     __shared__ uint32_t s_tile;
-    __shared__ uint32_t s_wave_count[kSortWaves][kRadix];
-    __shared__ uint32_t s_local_start[kRadix];
     __shared__ uint32_t s_global_delta[kRadix];
     __shared__ uint32_t s_scan_wave[kSortWaves];
-    __shared__ uint64_t s_keys[kSortTile];
-    __shared__ uint32_t s_vals[kSortTile];
+    // The ranking counters are dead once every pair knows its place in the tile,
+    // so they share LDS with the permutation buffer (51 KB: three workgroups per CU).
+    __shared__ __align__(16) unsigned char s_raw[kSortTile * 12];
+    uint32_t (*s_wave_count)[kRadix] = reinterpret_cast<uint32_t (*)[kRadix]>(s_raw);
+    uint32_t *s_local_start = reinterpret_cast<uint32_t *>(s_raw) + kSortWaves * kRadix;
+    uint64_t *s_keys = reinterpret_cast<uint64_t *>(s_raw);
+    uint32_t *s_vals = reinterpret_cast<uint32_t *>(s_raw + kSortTile * 8);
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -150,7 +174,15 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     }
 
     // Stable rank of each pair among the pairs of its wave with the same digit.
+    // Match: 8 ballots leave in `peers` the lanes that hold the same digit.  The
+    // lowest lane of each group adds the group size to the wave's counter row
+    // with a returning LDS atomic; LDS serves a wave's instructions in order, so
+    // item i sees the counts of items < i, and the 16 atomics are in flight
+    // together.  The group reads its leader's result with ds_bpermute.
     uint32_t *wave_row = s_wave_count[wave];
+    uint32_t below[kSortItems];
+    uint32_t leader[kSortItems];
+    uint32_t before[kSortItems];
 #pragma unroll
     for (int i = 0; i < kSortItems; i++) {
         const uint32_t d = (uint32_t)(key[i] >> shift) & (kRadix - 1);
@@ -161,14 +193,14 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
             const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
             peers &= bit ? vote : ~vote;
         }
-        const uint32_t below = lanes_below(peers);
-        const uint32_t group = (uint32_t)__builtin_popcountll(peers);
-        const uint32_t before = wave_row[d];
-        rank[i] = before + below;
-        __builtin_amdgcn_wave_barrier();
-        if (below == 0) wave_row[d] = before + group;
-        __builtin_amdgcn_wave_barrier();
+        below[i] = lanes_below(peers);
+        leader[i] = (uint32_t)__builtin_ctzll(peers);
+        before[i] = 0;
+        if (below[i] == 0) before[i] = __hip_atomic_fetch_add(wave_row + d, (uint32_t)__builtin_popcountll(peers), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+#pragma unroll
+    for (int i = 0; i < kSortItems; i++)
+        rank[i] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader[i] << 2), (int)before[i]) + below[i];
     __syncthreads();
 
     // Thread d owns digit d: per-wave exclusive offsets, tile count, look-back.
@@ -200,35 +232,55 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         s_local_start[tid] = wave_prefix + v - digit_count;
     }
 
+    // Place of every pair inside the tile, then permute into digit order in LDS
+    // (the buffer overlays the counters) and write digit runs contiguously.
+    const uint32_t local_start = s_local_start[tid];
+    __syncthreads();  // s_local_start is complete
+#pragma unroll
+    for (int i = 0; i < kSortItems; i++) {
+        const uint32_t d = (uint32_t)(key[i] >> shift) & (kRadix - 1);
+        rank[i] += s_local_start[d] + s_wave_count[wave][d];
+    }
+    __syncthreads();  // every pair knows its place: the counters may be overwritten
+#pragma unroll
+    for (int i = 0; i < kSortItems; i++) {
+        s_keys[rank[i]] = key[i];
+        s_vals[rank[i]] = val[i];
+    }
+    // While the pairs settle in LDS the predecessors publish their counts.
     uint32_t prefix = 0;
     bool timed_out = false;
-    for (int look = tile - 1; look >= 0; look--) {
-        uint32_t word = __hip_atomic_load(my_words + (size_t)look * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t spins = 0;
-        while ((word >> 30) == 0 && spins < kSortSpinLimit) {
-            __builtin_amdgcn_s_sleep(1);
-            word = __hip_atomic_load(my_words + (size_t)look * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            spins++;
+    for (int look = tile - 1; look >= 0 && !timed_out;) {
+        uint32_t words[kLookWindow];
+#pragma unroll
+        for (int k = 0; k < kLookWindow; k++)
+            words[k] = (look - k >= 0)
+                           ? __hip_atomic_load(my_words + (size_t)(look - k) * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                           : kLbInclusive;  // before the first tile: inclusive prefix 0
+        bool done = false;
+#pragma unroll
+        for (int k = 0; k < kLookWindow; k++) {
+            if (done || timed_out) continue;
+            uint32_t word = words[k];
+            uint32_t spins = 0;
+            while ((word >> 30) == 0 && spins < kSortSpinLimit) {
+                __builtin_amdgcn_s_sleep(1);
+                word = __hip_atomic_load(my_words + (size_t)(look - k) * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                spins++;
+            }
+            if ((word >> 30) == 0) { timed_out = true; continue; }
+            prefix += word & kLbValueMask;
+            if ((word >> 30) == 2) done = true;
         }
-        if ((word >> 30) == 0) { timed_out = true; break; }
-        prefix += word & kLbValueMask;
-        if ((word >> 30) == 2) break;
+        if (done) break;
+        look -= kLookWindow;
     }
     if (tile != 0)
         __hip_atomic_store(my_words + (size_t)tile * kRadix, kLbInclusive | ((prefix + published) & kLbValueMask), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     if (timed_out && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
-    s_global_delta[tid] = bases[tid] + prefix - s_local_start[tid];
-    __syncthreads();
+    s_global_delta[tid] = bases[tid] + prefix - local_start;
 
-    // Permute into digit order in LDS, then write digit runs contiguously.
-#pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
-        const uint32_t d = (uint32_t)(key[i] >> shift) & (kRadix - 1);
-        const uint32_t pos = s_local_start[d] + s_wave_count[wave][d] + rank[i];
-        s_keys[pos] = key[i];
-        s_vals[pos] = val[i];
-    }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < kSortItems; i++) {
@@ -261,11 +313,13 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
     }
     *result_in_alt = 0;
     hipStream_t s = (hipStream_t)stream;
-    if (status) {
-        TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
-        if (int e = check_launch("fill_zero_kernel")) return e;
+    if (n == 0 || end_bit == 0) {
+        if (status) {
+            TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
+            if (int e = check_launch("fill_zero_kernel")) return e;
+        }
+        return 0;
     }
-    if (n == 0 || end_bit == 0) return 0;
     if (!keys || !values || !keys_alt || !values_alt || !workspace) {
         set_error("tg_sort_pairs_u64_u32: null pointer");
         return TG_E_ARG;
@@ -285,17 +339,15 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
     uint32_t *partials = (uint32_t *)(ws + L.off_partials);
     uint32_t *lookback = (uint32_t *)(ws + L.off_lookback);
 
-    // tickets and look-back words start at zero; bases and partials are fully overwritten
-    TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, tickets, (size_t)64);
-    if (int e = check_launch("fill_zero_kernel")) return e;
-    const size_t lb_words = (size_t)L.passes * L.n_tiles * kRadix;
-    const int fill_blocks = (int)((lb_words + 1023) / 1024 < 2048 ? (lb_words + 1023) / 1024 : 2048);
-    TG_LAUNCH(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, lookback, lb_words);
+    // tickets and look-back words (adjacent) start at zero; bases and partials are fully overwritten
+    const size_t fill_words = 64 + (size_t)L.passes * L.n_tiles * kRadix;
+    const int fill_blocks = (int)((fill_words + 1023) / 1024 < 2048 ? (fill_words + 1023) / 1024 : 2048);
+    TG_LAUNCH(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, tickets, fill_words);
     if (int e = check_launch("fill_zero_kernel")) return e;
 
     TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials);
     if (int e = check_launch("sort_histogram_kernel")) return e;
-    TG_LAUNCH(sort_bases_kernel, dim3(L.passes), dim3(kSortThreads), 0, s, partials, L.hist_blocks, bases);
+    TG_LAUNCH(sort_bases_kernel, dim3(L.passes), dim3(kBasesThreads), 0, s, partials, L.hist_blocks, bases, status);
     if (int e = check_launch("sort_bases_kernel")) return e;
 
     uint64_t *kin = keys, *kout = keys_alt;
