@@ -67,10 +67,15 @@ int tg_bin_count(const float *vertices, int32_t n_vertices, const int32_t *indic
 /* Exclusive prefix sum of n uint32 (single pass, decoupled look-back).
  * out[i] = sum(in[0..i)), *total = sum(in[0..n)).  Replaces the
  * sum().item() / cumsum_out sequence of per_tile_lists (render.cu:290-295).
- * `status` (1 uint32, may be NULL) receives TG_STATUS_*; in and out may alias. */
+ * `status` (1 uint32, may be NULL) receives TG_STATUS_*; in and out may alias.
+ * Optional (heads may be NULL): for every h < head_capacity with
+ * h * head_stride < total, heads[h] = the index i whose output range
+ * [out[i], out[i] + in[i]) contains position h * head_stride.  tg_bin_emit uses
+ * it (head_stride 256) to find the triangle that owns a key without searching. */
 size_t tg_scan_workspace_bytes(int64_t n);
 int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
-                          size_t workspace_bytes, uint32_t *status, void *stream);
+                          size_t workspace_bytes, uint32_t *status, uint32_t head_stride, uint32_t head_capacity,
+                          uint32_t *heads, void *stream);
 
 /* Key emission: for triangle i and each tile of its AABB (tile x outer, tile y
  * inner, render.cu:235-236), at position tri_offsets[i] + local:
@@ -80,10 +85,12 @@ int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t
  * clipped to the tile (1e30 when the clip is empty) and orderable() is the
  * order-preserving map of float bits to uint32.  Replaces
  * fill_per_tile_lists_kernel, compute_plane, clip_polygon_to_halfspace
- * (render.cu:140-270).  n_keys = total of the scan. */
+ * (render.cu:140-270).  n_keys = total of the scan.  owner_heads (may be NULL)
+ * is the scan's `heads` output for head_stride = 256 with owner_capacity
+ * entries; without it the owners are found by binary search. */
 int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
-                int tile_h, const uint32_t *tri_offsets, int64_t n_keys, uint64_t *keys, uint32_t *payload,
-                void *stream);
+                int tile_h, const uint32_t *tri_offsets, int64_t n_keys, const uint32_t *owner_heads,
+                uint32_t owner_capacity, uint64_t *keys, uint32_t *payload, void *stream);
 
 /* ---- (2) radix sort --------------------------------------------------------- */
 

@@ -42,7 +42,7 @@ def test_host_side_helpers_and_argument_rejection():
     assert b"tg_bin_count" in lib.tg_last_error()
     assert lib.tg_bin_count(None, 3, None, 5, 64, 64, 16, 16, None, None) == -1
     assert lib.tg_bin_count(None, 0, None, 0, 64, 64, 16, 16, None, None) == 0  # nothing to do
-    assert lib.tg_scan_exclusive_u32(None, None, 8, None, None, 0, None, None) == -1
+    assert lib.tg_scan_exclusive_u32(None, None, 8, None, None, 0, None, 256, 0, None, None) == -1
     res = C.c_int(7)
     assert lib.tg_sort_pairs_u64_u32(None, None, None, None, 1 << 31, 64, None, 0, None, C.byref(res), None) == -1
     assert lib.tg_tile_ranges(None, 5, 10, None, None) == -1

@@ -75,6 +75,17 @@ def test_binning_sort_ranges_bit_exact(name, cuda, oracle):
     keys, payload = _C.bin_emit(d["vertices"], d["indices"], offs, K, W, H, tw, th)
     np.testing.assert_array_equal(u64(keys), em["keys64"])
     np.testing.assert_array_equal(payload.cpu().numpy(), em["tri"])
+    # same emission with the owners noted by the scan instead of searched, also with a table too short for all keys
+    for capacity in (_C.owner_heads_for(idx.shape[0], cuda).numel(), 3):
+        import torch
+        heads = torch.full((capacity,), -1, dtype=torch.int32, device=cuda)
+        offs2, total2, _ = _C.scan_exclusive(got_counts, heads=heads)
+        n_heads = min(capacity, -(-K // _C.OWNER_STRIDE))
+        want_heads = np.searchsorted(np.cumsum(tri_counts), np.arange(n_heads) * _C.OWNER_STRIDE, side="right")
+        np.testing.assert_array_equal(heads.cpu().numpy()[:n_heads], want_heads)
+        keys2, payload2 = _C.bin_emit(d["vertices"], d["indices"], offs2, K, W, H, tw, th, heads)
+        np.testing.assert_array_equal(u64(keys2), em["keys64"])
+        np.testing.assert_array_equal(payload2.cpu().numpy(), em["tri"])
 
     want_keys, want_vals = oracle.sort_pairs_u64(em["keys64"], em["tri"])
     skeys, svals, sstatus = _C.sort_pairs(keys, payload, _C.key_bits(T))

@@ -56,8 +56,15 @@ def bin_count(vertices, indices, width, height, tile_width, tile_height):
     return counts
 
 
-def scan_exclusive(counts, out=None):
-    """Exclusive prefix sum of an int32 tensor -> (offsets, total (1,) int32, status (1,) int32)."""
+OWNER_STRIDE = 256  # keys per workgroup of the emission kernel
+
+
+def scan_exclusive(counts, out=None, heads=None):
+    """Exclusive prefix sum of an int32 tensor -> (offsets, total (1,) int32, status (1,) int32).
+
+    heads (optional int32 tensor): receives, for every multiple of OWNER_STRIDE
+    below the total, the index of the element that owns that output position.
+    """
     _need_cuda(counts)
     lib = _lib.load()
     n = counts.numel()
@@ -68,12 +75,18 @@ def scan_exclusive(counts, out=None):
     ws_bytes = int(lib.tg_scan_workspace_bytes(n))
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(lib.tg_scan_exclusive_u32(_ptr(counts), _ptr(out), n, _ptr(total), _ptr(ws), ws_bytes, _ptr(status),
-                                             _stream(counts)), "tg_scan_exclusive_u32")
+        _lib.check(lib.tg_scan_exclusive_u32(_ptr(counts), _ptr(out), n, _ptr(total), _ptr(ws), ws_bytes, _ptr(status), OWNER_STRIDE,
+                                             0 if heads is None else heads.numel(), _ptr(heads), _stream(counts)),
+                   "tg_scan_exclusive_u32")
     return out, total, status
 
 
-def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, tile_height):
+def owner_heads_for(n_triangles, device):
+    """Buffer for the scan's `heads` output; covers up to 8 keys per triangle (beyond that the emission searches)."""
+    return torch.empty(((8 * n_triangles + 65536) // OWNER_STRIDE,), dtype=torch.int32, device=device)
+
+
+def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, tile_height, heads=None):
     """-> (keys (K,) int64 holding uint64 bit patterns, payload (K,) int32) in emission order."""
     _need_cuda(vertices, indices, tri_offsets)
     lib = _lib.load()
@@ -82,8 +95,8 @@ def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, 
     payload = torch.empty((n_keys,), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(lib.tg_bin_emit(_ptr(vertices), vertices.shape[0], _ptr(indices), indices.shape[0], width, height, tile_width,
-                                   tile_height, _ptr(tri_offsets), n_keys, _ptr(keys), _ptr(payload), _stream(vertices)),
-                   "tg_bin_emit")
+                                   tile_height, _ptr(tri_offsets), n_keys, _ptr(heads), 0 if heads is None else heads.numel(),
+                                   _ptr(keys), _ptr(payload), _stream(vertices)), "tg_bin_emit")
     return keys, payload
 
 
@@ -144,12 +157,13 @@ def per_tile_lists(vertices, indices, width, height, tile_width, tile_height):
     """
     T = num_tiles(width, height, tile_width, tile_height)
     counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
-    tri_offsets, total, status = scan_exclusive(counts, out=counts)
+    heads = owner_heads_for(indices.shape[0], vertices.device)
+    tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
     host = torch.stack([total[0], status[0]]).cpu()  # the one device->host read of the forward pass
     K, st = int(host[0]), int(host[1])
     if st != 0:
         raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
-    keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height)
+    keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
     keys, payload, sort_status = sort_pairs(keys, payload, key_bits(T))
     offsets = tile_ranges(keys, T)
     return payload, offsets, keys, sort_status
@@ -207,12 +221,13 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
         counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
-        tri_offsets, total, status = scan_exclusive(counts, out=counts)
+        heads = owner_heads_for(indices.shape[0], dev)
+        tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
         host = torch.stack([total[0], status[0]]).cpu()
         K, st = int(host[0]), int(host[1])
         if st != 0:
             raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
-        keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height)
+        keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
 
         timer.start("sorting")
         keys, sorted_ids, sort_status = sort_pairs(keys, payload, key_bits(T))

@@ -44,15 +44,21 @@ __global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const float4 *__
 
 // Per-thread polygon storage in LDS, slot-major so that lanes never conflict.
 constexpr int kPolyCap = 8;
+constexpr int kOwnerWindow = 1024;  // triangle offsets staged per workgroup for the owner search
 struct PolyLds {
     float x[2][kPolyCap][kBinThreads];
     float y[2][kPolyCap][kBinThreads];
 };
 
 // One Sutherland-Hodgman pass (render.cu:159-189) from buffer `src` to `1-src`
-// against nx*x + ny*y - d >= 0.  Returns the new vertex count.
-__device__ __forceinline__ int clip_pass(PolyLds &lds, int src, int n_in, float nx, float ny, float d) {
+// against nx*x + ny*y - d >= 0.  Returns the new vertex count.  When every
+// vertex is inside, the pass reproduces its input; `src` then stays current
+// (signalled by leaving it unchanged) and no vertex is copied.
+__device__ __forceinline__ int clip_pass(PolyLds &lds, int &src, int n_in, float nx, float ny, float d) {
     const int tid = threadIdx.x;
+    bool all_in = true;
+    for (int i = 0; i < n_in; i++) all_in = all_in && (nx * lds.x[src][i][tid] + ny * lds.y[src][i][tid] - d >= 0.0f);
+    if (all_in) return n_in;
     const int dst = 1 - src;
     int n_out = 0;
     float p0x = lds.x[src][n_in - 1][tid], p0y = lds.y[src][n_in - 1][tid];
@@ -78,6 +84,7 @@ __device__ __forceinline__ int clip_pass(PolyLds &lds, int src, int n_in, float 
         }
         p0x = p1x; p0y = p1y; d0 = d1; in0 = in1;
     }
+    src = dst;
     return n_out;
 }
 
@@ -95,14 +102,48 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__r
                                                                const int32_t *__restrict__ indices, int n_triangles, int W,
                                                                int H, int tw, int th, int tiles_x, int tiles_y,
                                                                const uint32_t *__restrict__ tri_offsets, int64_t n_keys,
+                                                               const uint32_t *__restrict__ owner_heads, uint32_t owner_capacity,
                                                                uint64_t *__restrict__ keys, uint32_t *__restrict__ payload) {
     __shared__ PolyLds lds;
+    __shared__ uint32_t s_offsets[kOwnerWindow];
     const int tid = threadIdx.x;
-    const int64_t k = (int64_t)blockIdx.x * kBinThreads + tid;
-    if (k >= n_keys) return;  // no barrier below: the LDS arrays are private per thread
+    const int64_t k0 = (int64_t)blockIdx.x * kBinThreads;
+    const int64_t k = k0 + tid;
+    // The owners of this workgroup's 256 keys lie between the owner of its first
+    // key and the owner of the next workgroup's first key; the scan noted both
+    // (otherwise two workgroup-uniform binary searches find them).  The offsets
+    // in between are staged in LDS and searched there.
+    int t_first, t_last;
+    if (owner_heads && blockIdx.x < owner_capacity) {
+        t_first = (int)owner_heads[blockIdx.x];
+        t_last = (k0 + kBinThreads < n_keys && blockIdx.x + 1 < owner_capacity) ? (int)owner_heads[blockIdx.x + 1] : n_triangles - 1;
+    } else {
+        const int64_t k_last = (k0 + kBinThreads <= n_keys ? k0 + kBinThreads : n_keys) - 1;
+        t_first = owner_of_key(tri_offsets, n_triangles, (uint32_t)k0);
+        t_last = owner_of_key(tri_offsets, n_triangles, (uint32_t)k_last);
+    }
+    const int span = t_last - t_first + 1;
+    const bool windowed = span <= kOwnerWindow;
+    if (windowed)
+        for (int i = tid; i < span; i += kBinThreads) s_offsets[i] = tri_offsets[t_first + i];
+    __syncthreads();
+    if (k >= n_keys) return;  // no barrier below: the polygon arrays are private per thread
 
-    const int t = owner_of_key(tri_offsets, n_triangles, (uint32_t)k);
-    const uint32_t local = (uint32_t)k - tri_offsets[t];
+    int t;
+    uint32_t owner_offset;
+    if (windowed) {
+        int lo = 0, hi = span;  // s_offsets[lo] <= k, answer in [lo, hi)
+        while (hi - lo > 1) {
+            const int mid = lo + ((hi - lo) >> 1);
+            if (s_offsets[mid] <= (uint32_t)k) lo = mid; else hi = mid;
+        }
+        t = t_first + lo;
+        owner_offset = s_offsets[lo];
+    } else {
+        t = owner_of_key(tri_offsets, n_triangles, (uint32_t)k);
+        owner_offset = tri_offsets[t];
+    }
+    const uint32_t local = (uint32_t)k - owner_offset;
     const TriXYZ p = load_triangle(vertices, n_vertices, indices, t);
     const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
     const uint32_t ny = (uint32_t)(r.y1 - r.y0 + 1);
@@ -126,16 +167,17 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__r
     lds.x[0][1][tid] = p.bx; lds.y[0][1][tid] = p.by;
     lds.x[0][2][tid] = p.cx; lds.y[0][2][tid] = p.cy;
     int n = 3;
-    n = clip_pass(lds, 0, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
-    if (n > 0) n = clip_pass(lds, 1, n, -1.0f, 0.0f, -xmax);
-    if (n > 0) n = clip_pass(lds, 0, n, 0.0f, 1.0f, ymin);
-    if (n > 0) n = clip_pass(lds, 1, n, 0.0f, -1.0f, -ymax);
+    int cur = 0;  // buffer that holds the current polygon
+    n = clip_pass(lds, cur, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
+    if (n > 0) n = clip_pass(lds, cur, n, -1.0f, 0.0f, -xmax);
+    if (n > 0) n = clip_pass(lds, cur, n, 0.0f, 1.0f, ymin);
+    if (n > 0) n = clip_pass(lds, cur, n, 0.0f, -1.0f, -ymax);
 
     float key = kFarKey;  // render.cu:259
     if (n > 0) {
         float md = FLT_MAX;
         for (int i = 0; i < n; i++) {
-            const float pd = A * lds.x[0][i][tid] + B * lds.y[0][i][tid] + C;  // render.cu:154-157
+            const float pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
             md = (pd < md) ? pd : md;
         }
         key = md;
@@ -204,15 +246,16 @@ extern "C" int tg_bin_count(const float *vertices, int32_t n_vertices, const int
 }
 
 extern "C" int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
-                           int tile_h, const uint32_t *tri_offsets, int64_t n_keys, uint64_t *keys, uint32_t *payload,
-                           void *stream) {
+                           int tile_h, const uint32_t *tri_offsets, int64_t n_keys, const uint32_t *owner_heads,
+                           uint32_t owner_capacity, uint64_t *keys, uint32_t *payload, void *stream) {
     if (int e = check_geometry("tg_bin_emit", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
     if (n_keys < 0 || n_keys > 0xffffffffll) { set_error("tg_bin_emit: n_keys out of range"); return TG_E_ARG; }
     if (n_keys == 0) return 0;
     if (n_triangles == 0 || !tri_offsets || !keys || !payload) { set_error("tg_bin_emit: null pointer"); return TG_E_ARG; }
     TG_LAUNCH(bin_emit_kernel, dim3((unsigned)ceil_div64(n_keys, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
                        (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
-                       ceil_div(width, tile_w), ceil_div(height, tile_h), tri_offsets, n_keys, keys, payload);
+                       ceil_div(width, tile_w), ceil_div(height, tile_h), tri_offsets, n_keys, owner_heads, owner_capacity, keys,
+                       payload);
     return check_launch("bin_emit_kernel");
 }
 

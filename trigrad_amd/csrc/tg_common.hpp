@@ -64,7 +64,9 @@ __device__ __forceinline__ float clampf(float v, float lo, float hi) { return (v
 // the source makes the product and quotient double precision.
 __device__ __forceinline__ int tile_coord(float m, int extent, int tile, int ntiles) {
     float m1 = m + 1.0f;
-    double t = (((double)m1 * 0.5) * (double)extent) / (double)tile;
+    const double scaled = ((double)m1 * 0.5) * (double)extent;
+    // dividing by a power of two is an exact scaling, so the reciprocal gives the same double
+    const double t = ((tile & (tile - 1)) == 0) ? scaled * (1.0 / (double)tile) : scaled / (double)tile;
     return (int)clampf((float)t, 0.0f, (float)(ntiles - 1));
 }
 

@@ -41,7 +41,8 @@ __global__ void scan_init_kernel(uint32_t *ticket, uint64_t *states, int n_tiles
 
 __global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint32_t *__restrict__ in, uint32_t *out, int64_t n,
                                                                      uint32_t *total, uint32_t *ticket, uint64_t *states,
-                                                                     int n_tiles, uint32_t *status) {
+                                                                     int n_tiles, uint32_t *status, uint32_t head_stride,
+                                                                     uint32_t head_capacity, uint32_t *__restrict__ heads) {
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_wave_total[kScanThreads / kWave];
     __shared__ uint32_t s_tile_prefix;
@@ -112,6 +113,15 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint3
     uint32_t run = s_tile_prefix + s_wave_total[wave] + (incl - thread_sum);
     uint32_t y[4];
     for (int k = 0; k < 4; k++) { y[k] = run; run += x[k]; }
+    if (heads) {
+        // element i owns the output positions [y, y + x): note for every multiple of
+        // head_stride which element owns it (few elements own one, most own none)
+        for (int k = 0; k < 4; k++) {
+            if (x[k] == 0 || base + k >= n) continue;
+            const uint32_t first = (y[k] + head_stride - 1) / head_stride, last = (y[k] + x[k] - 1) / head_stride;
+            for (uint32_t h = first; h <= last && h < head_capacity; h++) heads[h] = (uint32_t)(base + k);
+        }
+    }
     if (base + 4 <= n) {
         *reinterpret_cast<uint4 *>(out + base) = make_uint4(y[0], y[1], y[2], y[3]);
     } else {
@@ -134,13 +144,18 @@ extern "C" size_t tg_scan_workspace_bytes(int64_t n) {
 }
 
 extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
-                                     size_t workspace_bytes, uint32_t *status, void *stream) {
+                                     size_t workspace_bytes, uint32_t *status, uint32_t head_stride, uint32_t head_capacity,
+                                     uint32_t *heads, void *stream) {
     if (n < 0 || !total || !workspace || (n > 0 && (!in || !out))) {
         set_error("tg_scan_exclusive_u32: null pointer or negative size");
         return TG_E_ARG;
     }
     if (((uintptr_t)in & 15) || ((uintptr_t)out & 15) || ((uintptr_t)workspace & 7)) {
         set_error("tg_scan_exclusive_u32: in/out must be 16-byte aligned, workspace 8-byte aligned");
+        return TG_E_ARG;
+    }
+    if (heads && head_stride == 0) {
+        set_error("tg_scan_exclusive_u32: head_stride must be positive when heads is given");
         return TG_E_ARG;
     }
     if (n > (int64_t)kScanTile * 0x7fffffff / 2) {
@@ -160,6 +175,6 @@ extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t 
     if (int e = check_launch("scan_init_kernel")) return e;
     if (n_tiles == 0) return 0;
     TG_LAUNCH(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
-                       n_tiles, status);
+                       n_tiles, status, head_stride, head_capacity, heads);
     return check_launch("scan_lookback_kernel");
 }
