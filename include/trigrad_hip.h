@@ -152,6 +152,24 @@ int tg_render_backward(const float *grad_image, const float *grad_depthmap, cons
                        int per_pixel_sort, int max_layers, float *grad_vertices, float *grad_colors,
                        float *grad_opacities, void *stream);
 
+/* ---- host-side component hooks ---------------------------------------------- */
+
+/* HOST pointers, run on the CPU.  The reference exports the same six functions
+ * from its extension for its component tests (tests.cu:43-76: barycentric_torch,
+ * barycentric_backward_torch, interpolate3_scalar_torch, ..._backward_torch,
+ * interpolate3_vector_torch, ..._backward_torch around util.h:232-250, 299-355,
+ * 395-455).  2-vectors and 3-vectors are plain float arrays. */
+void tg_barycentric(const float *v0, const float *v1, const float *v2, const float *p, float *out3);
+void tg_barycentric_backward(const float *g3, const float *a, const float *b, const float *c, const float *p,
+                             float *grads_4x2);
+float tg_interpolate3_scalar(const float *bary, float a, float b, float c, const float *w);
+void tg_interpolate3_scalar_backward(float g, const float *bary, float a, float b, float c, const float *w,
+                                     float *grad_bary, float *grad_values, float *grad_w);
+void tg_interpolate3_vector(const float *bary, const float *a, const float *b, const float *c, const float *w, float *out3);
+void tg_interpolate3_vector_backward(const float *g3, const float *bary, const float *a, const float *b, const float *c,
+                                     const float *w, float *grad_bary, float *grad_a, float *grad_b, float *grad_c,
+                                     float *grad_w);
+
 #ifdef __cplusplus
 }
 #endif

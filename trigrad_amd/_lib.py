@@ -33,6 +33,12 @@ SIGNATURES = {
     "tg_bary": (_i, [_p, _i32, _p, _i32, _p, _p]),
     "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p]),
     "tg_render_backward": (_i, [_p] * 15 + [_i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p]),
+    "tg_barycentric": (None, [_p] * 5),
+    "tg_barycentric_backward": (None, [_p] * 6),
+    "tg_interpolate3_scalar": (_f, [_p, _f, _f, _f, _p]),
+    "tg_interpolate3_scalar_backward": (None, [_f, _p, _f, _f, _f, _p, _p, _p, _p]),
+    "tg_interpolate3_vector": (None, [_p] * 6),
+    "tg_interpolate3_vector_backward": (None, [_p] * 11),
 }
 
 _lib = None

@@ -17,7 +17,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtrigrad_hip.so")
 
-SOURCES = ["tg_api.hip", "tg_binning.hip", "tg_scan.hip", "tg_sort.hip", "tg_forward.hip", "tg_backward.hip"]
+SOURCES = ["tg_api.hip", "tg_binning.hip", "tg_scan.hip", "tg_sort.hip", "tg_forward.hip", "tg_backward.hip",
+           "tg_components.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
