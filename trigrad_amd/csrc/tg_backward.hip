@@ -306,10 +306,13 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     __shared__ float s_seed[kMaxWaves][kSeedWords][kWaveSlots];
     __shared__ float s_term[kMaxWaves][kTerms * kTermStride];
     __shared__ float s_px[kTileThreads], s_py[kTileThreads];
+    __shared__ uint8_t s_touch[kBackBatch];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
     __shared__ int s_last;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
+    const int n_waves = blockDim.x / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile];
     const PixelCoord p = pixel_of_thread(a);
@@ -321,6 +324,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     if (tid == 0) s_last = 0;
     s_px[tid] = p.px;
     s_py[tid] = p.py;
+    publish_wave_rect(p, s_rects);
     __syncthreads();
     const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
     if (my_last > 0) atomicMax(&s_last, my_last);
@@ -334,18 +338,26 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
         const int lo = max(0, hi - kBackBatch);
         const int nb = hi - lo;
         __syncthreads();  // every wave is done with the previous batch
-        for (int e = tid; e < nb; e += blockDim.x) gather_back(a, start + lo + e, s_rec[e]);
+        for (int e = tid; e < nb; e += blockDim.x) {
+            gather_back(a, start + lo + e, s_rec[e]);
+            s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+        }
         __syncthreads();
 
-        // 1. inside tests
+        // 1. inside tests, only for the entries that can touch this wave's pixels
         const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
         if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
+        ballots[lane] = 0;
+        ballots[lane + kWave] = 0;
+        wave_lds_sync();
         uint64_t m[2] = {0, 0};
 #pragma unroll
         for (int wd = 0; wd < 2; wd++) {
             uint64_t bits = 0;
-            const int count = min(64, nb - 64 * wd);
-            for (int bit = 0; bit < count; bit++) {
+            uint64_t todo = wave_candidates(s_touch, 64 * wd, nb, wave);
+            while (todo) {
+                const int bit = __builtin_ctzll(todo);
+                todo &= todo - 1;
                 const BackRecord &r = s_rec[64 * wd + bit];
                 float b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
@@ -483,10 +495,15 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     // flushed once per tile; positions beyond the window go straight to memory.
     float *s_acc = reinterpret_cast<float *>(tk.pos + kLayers * n_threads);
 
+    __shared__ uint8_t s_touch[kBatch];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
     const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int n_waves = blockDim.x / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
+    publish_wave_rect(p, s_rects);
     const int n_acc = min(end - start, kAccWindow);
     for (int i = tid; i < n_acc * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
 
@@ -509,10 +526,17 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
         for (int batch = start; batch < end; batch += kBatch) {
             const int nb = min(kBatch, end - batch);
             __syncthreads();
-            for (int e = tid; e < nb; e += blockDim.x) gather_depth(a, batch + e, s_rec[e]);
+            for (int e = tid; e < nb; e += blockDim.x) {
+                gather_depth(a, batch + e, s_rec[e]);
+                s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+            }
             __syncthreads();
-            if (want) {
-                for (int e = 0; e < nb; e++) {
+            for (int first = 0; first < nb; first += kWave) {
+                uint64_t todo = wave_candidates(s_touch, first, nb, wave);
+                while (todo) {
+                    const int e = first + __builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    if (!want) continue;
                     const DepthRecord &r = s_rec[e];
                     float b0, b1, b2;
                     bary_apply(r.m, p.px, p.py, b0, b1, b2);

@@ -44,10 +44,15 @@ __device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoor
 
 __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(RasterArgs a, ForwardOut out) {
     __shared__ BlendRecord s_rec[kBatch];
+    __shared__ uint8_t s_touch[kBatch];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
     const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int n_waves = blockDim.x / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
+    publish_wave_rect(p, s_rects);
 
     PixelState s;
     int last = 0;
@@ -55,17 +60,26 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         const bool running = p.valid && s.alpha > a.thr && s.blended < a.max_layers;
         if (!__syncthreads_or(running)) break;
         const int nb = min(kBatch, end - batch);
-        for (int e = tid; e < nb; e += blockDim.x) gather_blend(a, batch + e, s_rec[e]);
+        for (int e = tid; e < nb; e += blockDim.x) {
+            gather_blend(a, batch + e, s_rec[e]);
+            s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+        }
         __syncthreads();
-        if (running) {
-            for (int e = 0; e < nb; e++) {
-                if (!(s.alpha > a.thr && s.blended < a.max_layers)) break;  // render.cu:578
-                const BlendRecord &r = s_rec[e];
-                float b0, b1, b2;
-                bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                if (!bary_inside(b0, b1, b2)) continue;
-                blend_fragment(s, r, b0, b1, b2);
-                last = batch + e - start + 1;
+        // the wave walks only the entries that can touch its pixels, in list order
+        for (int first = 0; first < nb; first += kWave) {
+            uint64_t todo = wave_candidates(s_touch, first, nb, wave);
+            while (todo) {
+                const int e = first + __builtin_ctzll(todo);
+                todo &= todo - 1;
+                if (running && s.alpha > a.thr && s.blended < a.max_layers) {  // render.cu:578
+                    const BlendRecord &r = s_rec[e];
+                    float b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    if (bary_inside(b0, b1, b2)) {
+                        blend_fragment(s, r, b0, b1, b2);
+                        last = batch + e - start + 1;
+                    }
+                }
             }
         }
     }
@@ -95,10 +109,15 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
     tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
 
+    __shared__ uint8_t s_touch[kBatch];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
     const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int n_waves = blockDim.x / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
+    publish_wave_rect(p, s_rects);
 
     PixelState s;
     float last_depth = -__builtin_inff();  // render.cu:585-586
@@ -112,10 +131,17 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         for (int batch = start; batch < end; batch += kBatch) {
             const int nb = min(kBatch, end - batch);
             __syncthreads();
-            for (int e = tid; e < nb; e += blockDim.x) gather_depth(a, batch + e, s_rec[e]);
+            for (int e = tid; e < nb; e += blockDim.x) {
+                gather_depth(a, batch + e, s_rec[e]);
+                s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+            }
             __syncthreads();
-            if (want) {
-                for (int e = 0; e < nb; e++) {
+            for (int first = 0; first < nb; first += kWave) {
+                uint64_t todo = wave_candidates(s_touch, first, nb, wave);
+                while (todo) {
+                    const int e = first + __builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    if (!want) continue;
                     const DepthRecord &r = s_rec[e];
                     float b0, b1, b2;
                     bary_apply(r.m, p.px, p.py, b0, b1, b2);

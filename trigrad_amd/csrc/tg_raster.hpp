@@ -140,6 +140,71 @@ size_t pixel_order_lds_bytes(int n_threads);
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
 int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
 
+// ---- per-wave culling ------------------------------------------------------------------
+// A wave owns 64 pixels of the tile.  Before its lanes test a list entry, the
+// entry is tested once against the rectangle spanned by the wave's pixel
+// centres.  The test is exact, not approximate: every IEEE operation is monotone
+// in each operand, so the inside test's own expression m0*x + m1*y + m2,
+// evaluated with the same operations at the corner that maximises it, bounds
+// the value every pixel of the rectangle would compute.  If that bound is below
+// the inside threshold for one of the three coordinates, no lane can hit.
+struct WaveRect { float x_lo, x_hi, y_lo, y_hi; };
+
+__device__ __forceinline__ bool may_touch(const float m[9], const WaveRect &r) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        const float mx = m[3 * k], my = m[3 * k + 1];
+        const float x = (mx >= 0.0f) ? r.x_hi : r.x_lo;
+        const float y = (my >= 0.0f) ? r.y_hi : r.y_lo;
+        const float bound = mx * x + my * y + m[3 * k + 2];
+        if (bound < kEffZero) return false;  // a NaN bound never culls
+    }
+    return true;
+}
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+constexpr int kMaxTileWaves = kTileThreads / kWave;
+
+// Every wave publishes the rectangle of its valid pixels (an empty rectangle,
+// lo > hi, if it has none); call with all threads, followed by __syncthreads().
+__device__ __forceinline__ void publish_wave_rect(const PixelCoord &p, WaveRect *s_rects) {
+    const float big = 3.0e38f;
+    WaveRect r;
+    r.x_lo = wave_min(p.valid ? p.px : big);
+    r.x_hi = wave_max(p.valid ? p.px : -big);
+    r.y_lo = wave_min(p.valid ? p.py : big);
+    r.y_hi = wave_max(p.valid ? p.py : -big);
+    if ((threadIdx.x & (kWave - 1)) == 0) s_rects[threadIdx.x / kWave] = r;
+}
+
+// Bit w of the result: wave w has to look at the entry.
+__device__ __forceinline__ uint32_t waves_touched(const float m[9], const WaveRect *s_rects, int n_waves) {
+    uint32_t bits = 0;
+#pragma unroll 1
+    for (int w = 0; w < n_waves; w++) {
+        const WaveRect r = s_rects[w];
+        if (r.x_lo <= r.x_hi && may_touch(m, r)) bits |= 1u << w;
+    }
+    return bits;
+}
+
+// 64 staged entries starting at `first`: mask of those the calling wave has to look at.
+__device__ __forceinline__ uint64_t wave_candidates(const uint8_t *s_touch, int first, int n_entries, int wave) {
+    const int e = first + (threadIdx.x & (kWave - 1));
+    const bool mine = e < n_entries && ((s_touch[e] >> wave) & 1u);
+    return __builtin_amdgcn_ballot_w64(mine);
+}
+
 // Per-pixel candidate lists of the per-pixel-sort mode live in LDS, slot-major:
 // entry `slot` of thread `t` is at [slot * n_threads + t] (conflict-free).
 struct TopK {
