@@ -65,21 +65,40 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
             s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
         }
         __syncthreads();
-        // the wave walks only the entries that can touch its pixels, in list order
-        for (int first = 0; first < nb; first += kWave) {
-            uint64_t todo = wave_candidates(s_touch, first, nb, wave);
+        // 1. inside tests of the entries that can touch this wave's pixels: all lanes
+        //    look at the same record (LDS broadcast); a lane keeps its hits as a 256-bit mask
+        uint64_t m[kBatch / kWave];
+#pragma unroll
+        for (int wd = 0; wd < kBatch / kWave; wd++) {
+            uint64_t bits = 0;
+            uint64_t todo = wave_candidates(s_touch, wd * kWave, nb, wave);
             while (todo) {
-                const int e = first + __builtin_ctzll(todo);
+                const int bit = __builtin_ctzll(todo);
                 todo &= todo - 1;
-                if (running && s.alpha > a.thr && s.blended < a.max_layers) {  // render.cu:578
-                    const BlendRecord &r = s_rec[e];
-                    float b0, b1, b2;
-                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                    if (bary_inside(b0, b1, b2)) {
-                        blend_fragment(s, r, b0, b1, b2);
-                        last = batch + e - start + 1;
-                    }
-                }
+                const BlendRecord &r = s_rec[wd * kWave + bit];
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                if (bary_inside(b0, b1, b2)) bits |= 1ull << bit;
+            }
+            m[wd] = running ? bits : 0ull;
+        }
+        // 2. every lane composites its own hits in list order, so the blend arithmetic
+        //    runs with as many lanes busy as there are pixels with a fragment left
+        while (true) {
+            int e = -1;
+            if (s.alpha > a.thr && s.blended < a.max_layers) {  // render.cu:578, tested before every fragment
+                if (m[0]) { e = __builtin_ctzll(m[0]); m[0] &= m[0] - 1; }
+                else if (m[1]) { e = __builtin_ctzll(m[1]); m[1] &= m[1] - 1; e += 64; }
+                else if (m[2]) { e = __builtin_ctzll(m[2]); m[2] &= m[2] - 1; e += 128; }
+                else if (m[3]) { e = __builtin_ctzll(m[3]); m[3] &= m[3] - 1; e += 192; }
+            }
+            if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
+            if (e >= 0) {
+                const BlendRecord &r = s_rec[e];
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                blend_fragment(s, r, b0, b1, b2);
+                last = batch + e - start + 1;
             }
         }
     }
