@@ -531,20 +531,19 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
                 s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
             }
             __syncthreads();
-            for (int first = 0; first < nb; first += kWave) {
-                uint64_t todo = wave_candidates(s_touch, first, nb, wave);
-                while (todo) {
-                    const int e = first + __builtin_ctzll(todo);
-                    todo &= todo - 1;
-                    if (!want) continue;
-                    const DepthRecord &r = s_rec[e];
-                    float b0, b1, b2;
-                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                    if (!bary_inside(b0, b1, b2)) continue;
-                    const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
-                    const int j = batch + e;
-                    if (pd < bound_depth || (pd == bound_depth && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
-                }
+            uint64_t m[kBatch / kWave];
+            batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
+            if (!want) m[0] = m[1] = m[2] = m[3] = 0;
+            while (true) {
+                const int e = pop_lowest(m);
+                if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
+                if (e < 0) continue;
+                const DepthRecord &r = s_rec[e];
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
+                const int j = batch + e;
+                if (pd < bound_depth || (pd == bound_depth && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
             }
         }
         if (want) {

@@ -65,33 +65,15 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
             s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
         }
         __syncthreads();
-        // 1. inside tests of the entries that can touch this wave's pixels: all lanes
-        //    look at the same record (LDS broadcast); a lane keeps its hits as a 256-bit mask
+        // 1. inside tests; a lane keeps its hits as a 256-bit mask
         uint64_t m[kBatch / kWave];
-#pragma unroll
-        for (int wd = 0; wd < kBatch / kWave; wd++) {
-            uint64_t bits = 0;
-            uint64_t todo = wave_candidates(s_touch, wd * kWave, nb, wave);
-            while (todo) {
-                const int bit = __builtin_ctzll(todo);
-                todo &= todo - 1;
-                const BlendRecord &r = s_rec[wd * kWave + bit];
-                float b0, b1, b2;
-                bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                if (bary_inside(b0, b1, b2)) bits |= 1ull << bit;
-            }
-            m[wd] = running ? bits : 0ull;
-        }
+        batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
+        if (!running) m[0] = m[1] = m[2] = m[3] = 0;
         // 2. every lane composites its own hits in list order, so the blend arithmetic
         //    runs with as many lanes busy as there are pixels with a fragment left
         while (true) {
             int e = -1;
-            if (s.alpha > a.thr && s.blended < a.max_layers) {  // render.cu:578, tested before every fragment
-                if (m[0]) { e = __builtin_ctzll(m[0]); m[0] &= m[0] - 1; }
-                else if (m[1]) { e = __builtin_ctzll(m[1]); m[1] &= m[1] - 1; e += 64; }
-                else if (m[2]) { e = __builtin_ctzll(m[2]); m[2] &= m[2] - 1; e += 128; }
-                else if (m[3]) { e = __builtin_ctzll(m[3]); m[3] &= m[3] - 1; e += 192; }
-            }
+            if (s.alpha > a.thr && s.blended < a.max_layers) e = pop_lowest(m);  // render.cu:578, tested before every fragment
             if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
             if (e >= 0) {
                 const BlendRecord &r = s_rec[e];
@@ -155,22 +137,23 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
             }
             __syncthreads();
-            for (int first = 0; first < nb; first += kWave) {
-                uint64_t todo = wave_candidates(s_touch, first, nb, wave);
-                while (todo) {
-                    const int e = first + __builtin_ctzll(todo);
-                    todo &= todo - 1;
-                    if (!want) continue;
-                    const DepthRecord &r = s_rec[e];
-                    float b0, b1, b2;
-                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                    if (!bary_inside(b0, b1, b2)) continue;
-                    const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
-                    const int j = batch + e;
-                    if (pd < last_depth) continue;
-                    if (pd == last_depth && j <= last_j) continue;
-                    topk_insert(tk, cap, found, pd, j);
-                }
+            // inside tests into a per-lane mask, then every lane visits its own hits in
+            // list order (the order insert_sorted_topk sees them in the reference)
+            uint64_t m[kBatch / kWave];
+            batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
+            if (!want) m[0] = m[1] = m[2] = m[3] = 0;
+            while (true) {
+                const int e = pop_lowest(m);
+                if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
+                if (e < 0) continue;
+                const DepthRecord &r = s_rec[e];
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
+                const int j = batch + e;
+                if (pd < last_depth) continue;
+                if (pd == last_depth && j <= last_j) continue;
+                topk_insert(tk, cap, found, pd, j);
             }
         }
         if (want) {

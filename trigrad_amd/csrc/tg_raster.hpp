@@ -205,6 +205,39 @@ __device__ __forceinline__ uint64_t wave_candidates(const uint8_t *s_touch, int 
     return __builtin_amdgcn_ballot_w64(mine);
 }
 
+// Inside tests of one staged batch for the calling lane's pixel: bit e of the
+// result (word e / 64) is set when record e covers the pixel.  All lanes of the
+// wave read the same record at the same time (LDS broadcast); only records that
+// can touch the wave's pixels are looked at.  Rec must have a member m[9].
+template <typename Rec>
+__device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *s_touch, int nb, int wave, float px, float py,
+                                               uint64_t m[kBatch / kWave]) {
+#pragma unroll
+    for (int wd = 0; wd < kBatch / kWave; wd++) {
+        uint64_t bits = 0;
+        uint64_t todo = wave_candidates(s_touch, wd * kWave, nb, wave);
+        while (todo) {
+            const int bit = __builtin_ctzll(todo);
+            todo &= todo - 1;
+            float b0, b1, b2;
+            bary_apply(s_rec[wd * kWave + bit].m, px, py, b0, b1, b2);
+            if (bary_inside(b0, b1, b2)) bits |= 1ull << bit;
+        }
+        m[wd] = bits;
+    }
+}
+
+// Lowest set bit of a 256-bit mask, removed from the mask; -1 if the mask is empty.
+__device__ __forceinline__ int pop_lowest(uint64_t m[kBatch / kWave]) {
+    static_assert(kBatch / kWave == 4, "four 64-bit words");
+    int e = -1;
+    if (m[0]) { e = __builtin_ctzll(m[0]); m[0] &= m[0] - 1; }
+    else if (m[1]) { e = 64 + __builtin_ctzll(m[1]); m[1] &= m[1] - 1; }
+    else if (m[2]) { e = 128 + __builtin_ctzll(m[2]); m[2] &= m[2] - 1; }
+    else if (m[3]) { e = 192 + __builtin_ctzll(m[3]); m[3] &= m[3] - 1; }
+    return e;
+}
+
 // Per-pixel candidate lists of the per-pixel-sort mode live in LDS, slot-major:
 // entry `slot` of thread `t` is at [slot * n_threads + t] (conflict-free).
 struct TopK {
