@@ -30,6 +30,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of sort_sweep_kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
+# 256 MiB plain copy (profiles/config2_hbm_traffic_counters.md), keyed by the number of pairs it was measured on.
+MEASURED_SWEEP_TRAFFIC = {2186877: 61.0e6}
+
 MODES = {
     "A": dict(per_pixel_sort=True, max_layers=32),    # API defaults
     "B": dict(per_pixel_sort=False, max_layers=-1),   # tile-order compositing, early termination, full reverse traversal
@@ -46,6 +50,8 @@ def main():
     ap.add_argument("--sort-keys", type=int, default=10_000_000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain device copies of 256 MiB (a known traffic, for scaling rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -89,6 +95,14 @@ def main():
 
     ms = timed(lambda: step(args.mode), args.steps, args.warmup)
 
+    if args.calibrate_copy:
+        src = torch.empty((64 << 20,), dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- per-kernel durations from events on the launch stream -------------------
     _C.profile_enable(True)
     _C.profile_report()
@@ -129,7 +143,7 @@ def main():
                                f"per_pixel_sort={MODES[args.mode]['per_pixel_sort']}, max_layers={MODES[args.mode]['max_layers']}",
                    "mode": args.mode},
         "roofline": {"bound": "hbm", "kernel": "sort_sweep_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_SWEEP_TRAFFIC.get(K),
                      "bytes_per_launch": sweep_bytes, "avg_launch_us": sweep_avg_s * 1e6},
     }
 
