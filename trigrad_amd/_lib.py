@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtrigrad_hip.so")
+# TRIGRAD_HIP_LIB names another build of the same library (same ABI), e.g. one made with different tuning constants
+LIB_PATH = os.environ.get("TRIGRAD_HIP_LIB") or os.path.join(_HERE, "lib", "libtrigrad_hip.so")
 
 _p = C.c_void_p
 _i = C.c_int

@@ -161,13 +161,20 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 active = false;  // render.cu:594
             } else {
                 const int todo = min(found, a.max_layers - s.blended);
-                for (int i = 0; i < todo; i++) {
-                    BlendRecord r;
-                    gather_blend(a, tk.j(i), r);
-                    float b0, b1, b2;
-                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                    if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
-                    blend_fragment(s, r, b0, b1, b2);
+                // kGatherAhead records are fetched together: their chains of dependent
+                // loads (list -> indices -> vertices) overlap instead of adding up
+                for (int i0 = 0; i0 < todo; i0 += kGatherAhead) {
+                    BlendRecord r[kGatherAhead];
+#pragma unroll
+                    for (int u = 0; u < kGatherAhead; u++) gather_blend(a, tk.j(min(i0 + u, todo - 1)), r[u]);
+#pragma unroll
+                    for (int u = 0; u < kGatherAhead; u++) {
+                        if (i0 + u >= todo) break;
+                        float b0, b1, b2;
+                        bary_apply(r[u].m, p.px, p.py, b0, b1, b2);
+                        if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
+                        blend_fragment(s, r[u], b0, b1, b2);
+                    }
                 }
                 last_depth = tk.d(todo - 1);
                 last_j = tk.j(todo - 1);

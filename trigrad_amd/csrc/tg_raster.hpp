@@ -17,6 +17,7 @@ constexpr int kBatch = 256;         // list entries staged per batch
 constexpr int kLayers = 32;         // per-pixel selection batch (render.cu:570, :655)
 constexpr int kMaxTilePixels = 1024;  // tile_w * tile_h limit of the API (wrapper.py:143)
 constexpr int kTileThreads = 256;     // workgroup size limit
+constexpr int kGatherAhead = 4;       // records a lane of a per-pixel-order kernel fetches together
 
 struct RasterArgs {
     const float4 *vertices;
