@@ -35,6 +35,8 @@ extern "C" {
 #define TG_E_WORKSPACE (-2) /* workspace too small */
 
 /* Status word values written by the kernels that wait on other workgroups. */
+#define TG_MAX_SAVED_LAYERS 32 /* largest max_layers for which the forward pass can save the blend order */
+
 #define TG_STATUS_OK 0u
 #define TG_STATUS_LOOKBACK_TIMEOUT 1u
 
@@ -131,26 +133,33 @@ int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, i
  * blended entry, and last_depth (H,W) = that entry's pixel depth when
  * per_pixel_sort is on (render.cu:605-606 lastJ / lastDepth).  last and
  * last_depth may be NULL; the backward pass needs them.
+ * fragments (max_layers,H,W) int32, or NULL: with per_pixel_sort and
+ * max_layers <= TG_MAX_SAVED_LAYERS the kernel also writes, for every pixel,
+ * the list positions (relative to the tile's start) of its blended fragments
+ * in blend order (layer k of pixel p at fragments[k*H*W + p], k < ends[p]);
+ * tg_render_backward then walks them backwards instead of selecting the
+ * fragments again (the reference re-selects, render.cu:667-693).
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
 int tg_render_forward(const float *vertices, const int32_t *indices, const float *colors, const float *opacities,
                       const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
                       int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
                       float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
-                      float *last_depth, void *stream);
+                      float *last_depth, int32_t *fragments, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
 
 /* Accumulates into grad_vertices (V,4), grad_colors (V,3), grad_opacities (V),
  * which the caller zero-initialises.  Replaces render_backward_kernel /
  * process_backward (render.cu:455-538, 621-695).  Fragments are visited in
- * exact reverse blend order. */
+ * exact reverse blend order.  fragments: what tg_render_forward saved, or NULL
+ * (then last and, with per_pixel_sort, last_depth locate the far end). */
 int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
                        const int32_t *indices, const float *colors, const float *opacities,
                        const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
                        const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
-                       const float *last_depth, int width, int height, int tile_w, int tile_h, float early_stopping_threshold,
-                       int per_pixel_sort, int max_layers, float *grad_vertices, float *grad_colors,
-                       float *grad_opacities, void *stream);
+                       const float *last_depth, const int32_t *fragments, int width, int height, int tile_w, int tile_h,
+                       float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
+                       float *grad_colors, float *grad_opacities, void *stream);
 
 /* ---- host-side component hooks ---------------------------------------------- */
 

@@ -48,7 +48,7 @@ def _forward_both(scene, tw, th, mode, cuda, oracle, thr=1 / 256):
 
 
 def _check_forward(name, want, got):
-    image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status) = got
+    image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status, fragments) = got
     assert int(status.item()) == 0
     np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
     np.testing.assert_array_equal(sorted_ids.cpu().numpy(), want["sorted_ids"])
@@ -62,6 +62,18 @@ def _check_forward(name, want, got):
     assert_close(f"{name}: depthmap", np.where(fin, dm, 0), np.where(fin, want["depthmap"], 0), 1e-5, 1e-5)
     np.testing.assert_array_equal(ends.cpu().numpy(), want["ends"])
     np.testing.assert_array_equal(last.cpu().numpy(), want["last"])
+    if fragments is not None:
+        # saved blend order: `ends` valid layers per pixel, no list position twice, and the last
+        # layer is the entry `last` points at (the backward parity tests check the content)
+        fr = fragments.cpu().numpy()
+        en, la = want["ends"], want["last"]
+        layer = np.arange(fr.shape[0])[:, None, None]
+        valid = layer < en[None]
+        assert (fr[valid] >= 0).all()
+        ys, xs = np.nonzero(en > 0)
+        np.testing.assert_array_equal(fr[en[ys, xs] - 1, ys, xs], la[ys, xs] - 1)
+        srt = np.sort(np.where(valid, fr, -1 - layer), axis=0)
+        assert (np.diff(srt, axis=0) != 0).all()
     # (NaN results carry different payload/sign bits on the two machines)
     differing = int(((img.view(np.uint32) != want["image"].view(np.uint32)) & ~np.isnan(img)).sum())
     assert differing == 0, f"{name}: {differing} image values are not bit-identical to the oracle"
@@ -104,17 +116,24 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
     gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
                                         W, H, tw, th, m["per_pixel_sort"], ml, literal=False)
     image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
-    out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
-                             d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H, tw, th,
-                             1 / 256, m["per_pixel_sort"], ml, resume=resume)
-    for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
-        g = g.cpu().numpy().astype(np.float64)
-        # float32 summation of n terms: allow rtol on the result plus the rounding
-        # of the largest partial sums (scale of the gradient array)
-        scale = float(np.nanmax(np.abs(w))) if w.size else 0.0
-        assert_close(f"{name}/{mode}: {label}", np.nan_to_num(g), np.nan_to_num(w), GRAD_RTOL, GRAD_ATOL + 2e-6 * scale)
-        assert np.array_equal(np.isnan(g), np.isnan(w))
-    assert float(out[0][:, 2].abs().max()) == 0.0  # z never receives a gradient (render.cu:531-533)
+    # the blend order is saved exactly when per-pixel order meets max_layers <= 32;
+    # then the route that selects the fragments again is checked as well
+    saved_order = resume[3] is not None
+    assert saved_order == (bool(m["per_pixel_sort"]) and ml <= _C.MAX_SAVED_LAYERS)
+    routes = [("", resume)] + ([(" (re-selected)", resume[:3] + (None,))] if saved_order else [])
+    for route, res in routes:
+        out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
+                                 d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H,
+                                 tw, th, 1 / 256, m["per_pixel_sort"], ml, resume=res)
+        for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
+            g = g.cpu().numpy().astype(np.float64)
+            # float32 summation of n terms: allow rtol on the result plus the rounding
+            # of the largest partial sums (scale of the gradient array)
+            scale = float(np.nanmax(np.abs(w))) if w.size else 0.0
+            assert_close(f"{name}/{mode}{route}: {label}", np.nan_to_num(g), np.nan_to_num(w), GRAD_RTOL,
+                         GRAD_ATOL + 2e-6 * scale)
+            assert np.array_equal(np.isnan(g), np.isnan(w))
+        assert float(out[0][:, 2].abs().max()) == 0.0  # z never receives a gradient (render.cu:531-533)
 
 
 def test_default_mode_literal_and_policy_agree(oracle):

@@ -57,6 +57,11 @@ def bin_count(vertices, indices, width, height, tile_width, tile_height):
 
 
 OWNER_STRIDE = 256  # keys per workgroup of the emission kernel
+MAX_SAVED_LAYERS = 32  # TG_MAX_SAVED_LAYERS of the C header
+# With per_pixel_sort and max_layers <= MAX_SAVED_LAYERS the forward pass saves every pixel's
+# blend order ((max_layers, H, W) int32) and the backward pass walks it in reverse instead of
+# selecting the fragments again.  False trades the memory for the re-selection.
+SAVE_BLEND_ORDER = True
 
 
 def scan_exclusive(counts, out=None, heads=None):
@@ -198,8 +203,9 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
     """Reference _C.render_forward (render.cu:713-763).
 
     -> (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume)
-    `resume` = (last, last_depth, status): what the backward pass needs to start
-    its reverse traversal, plus the sort's status word.
+    `resume` = (last, last_depth, status, fragments): what the backward pass needs
+    for its reverse traversal (fragments is None unless the blend order was saved),
+    plus the sort's status word.
     """
     _need_cuda(vertices, indices, colors, opacities)
     lib = _lib.load()
@@ -217,6 +223,8 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         ends = torch.empty((height, width), dtype=torch.int32, device=dev)
         last = torch.empty((height, width), dtype=torch.int32, device=dev)
         last_depth = torch.empty((height, width), dtype=torch.float32, device=dev) if per_pixel_sort else None
+        save_order = bool(per_pixel_sort) and SAVE_BLEND_ORDER and 0 < int(max_layers) <= MAX_SAVED_LAYERS
+        fragments = torch.empty((int(max_layers), height, width), dtype=torch.int32, device=dev) if save_order else None
 
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
@@ -240,10 +248,11 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         _lib.check(lib.tg_render_forward(
             _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
             width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
-            _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _stream(vertices)),
-            "tg_render_forward")
+            _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
+            _stream(vertices)), "tg_render_forward")
         timings = timer.stop()
-    return image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, (last, last_depth, sort_status)
+    return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
+            (last, last_depth, sort_status, fragments))
 
 
 def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
@@ -252,7 +261,7 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
     """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities)."""
     if resume is None:
         raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
-    last, last_depth, sort_status = resume
+    last, last_depth, sort_status, fragments = resume
     _need_cuda(grad_output, vertices)
     lib = _lib.load()
     dev = vertices.device
@@ -263,7 +272,7 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
         grad_colors = torch.zeros_like(tensors[4])
         grad_opacities = torch.zeros_like(tensors[5])
         _lib.check(lib.tg_render_backward(
-            *[_ptr(t) for t in tensors], _ptr(last_depth), width, height, tile_width, tile_height,
+            *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
             _ptr(grad_opacities), _stream(vertices)), "tg_render_backward")
     return grad_vertices, grad_colors, grad_opacities

@@ -28,6 +28,7 @@ struct BackwardArgs {
     const int32_t *ends;
     const int32_t *last;
     const float *last_depth;
+    const int32_t *fragments;  // saved by the forward pass, or null
     float *grad_vertices;
     float *grad_colors;
     float *grad_opacities;
@@ -586,6 +587,79 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     }
 }
 
+// Per-pixel order with the blend order saved by the forward pass
+// (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  The records of the first
+// kSavedWindow list entries of the tile are staged once (rows an odd number of
+// words apart, so lanes reading different entries use different banks) and the
+// gradient sums of those entries are kept in LDS; later entries are gathered
+// from and added to memory directly.
+constexpr int kSavedWindow = 256;
+constexpr int kBackWords = (int)(sizeof(BackRecord) / sizeof(float));  // 36
+constexpr int kSavedStride = kBackWords + 1;
+
+__global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
+    __shared__ float s_rows[kSavedWindow * kSavedStride];
+    __shared__ float s_acc[kSavedWindow * kTerms];
+    const int tid = threadIdx.x;
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int start = a.offsets[tile], end = a.offsets[tile + 1];
+    const PixelCoord p = pixel_of_thread(a);
+    const int n_win = min(end - start, kSavedWindow);
+    for (int e = tid; e < n_win; e += blockDim.x) {
+        BackRecord r;
+        gather_back(a, start + e, r);
+        const float *w = reinterpret_cast<const float *>(&r);
+#pragma unroll
+        for (int k = 0; k < kBackWords; k++) s_rows[e * kSavedStride + k] = w[k];
+    }
+    for (int i = tid; i < n_win * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
+    __syncthreads();
+
+    if (p.valid) {
+        BackState st = load_back_state(g, p);
+        const int n = min(g.ends[p.index], a.max_layers);  // render.cu:642
+        const int64_t plane = (int64_t)a.W * a.H;
+        for (int hi = n; hi > 0; hi -= kGatherAhead) {
+            int rel[kGatherAhead];
+#pragma unroll
+            for (int u = 0; u < kGatherAhead; u++) rel[u] = g.fragments[(int64_t)max(hi - 1 - u, 0) * plane + p.index];
+#pragma unroll
+            for (int u = 0; u < kGatherAhead; u++) {
+                if (hi - 1 - u < 0) break;
+                BackRecord r;
+                if (rel[u] < n_win) {
+                    float *w = reinterpret_cast<float *>(&r);
+#pragma unroll
+                    for (int k = 0; k < kBackWords; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
+                } else {
+                    gather_back(a, start + rel[u], r);
+                }
+                float b0, b1, b2;
+                bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                float term[kTerms];
+                fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
+                if (rel[u] < n_win) {
+#pragma unroll
+                    for (int q = 0; q < kTerms; q++) atomicAdd(s_acc + rel[u] * kTerms + q, term[q]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < kTerms; q++)
+                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < n_win; e += blockDim.x) {
+        const int *id = reinterpret_cast<const int *>(s_rows + e * kSavedStride + (kBackWords - 3));
+#pragma unroll
+        for (int q = 0; q < kTerms; q++) {
+            const float v = s_acc[e * kTerms + q];
+            if (v != 0.0f) unsafeAtomicAdd(term_address(g, id[q / 7], q % 7), v);
+        }
+    }
+}
+
 size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads) + (size_t)kAccWindow * kTerms * sizeof(float); }
 
 }  // namespace tg
@@ -596,13 +670,13 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
                                   const int32_t *indices, const float *colors, const float *opacities,
                                   const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
                                   const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
-                                  const float *last_depth, int width, int height, int tile_w, int tile_h,
-                                  float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
+                                  const float *last_depth, const int32_t *fragments, int width, int height, int tile_w,
+                                  int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
                                   float *grad_colors, float *grad_opacities, void *stream) {
     if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!grad_image || !grad_depthmap || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
         !depthmap || !final_weights || !ends || !last || !grad_vertices || !grad_colors || !grad_opacities ||
-        (per_pixel_sort && !last_depth)) {
+        (per_pixel_sort && !last_depth && !fragments)) {
         set_error("tg_render_backward: null pointer");
         return TG_E_ARG;
     }
@@ -613,12 +687,21 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
     RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
     BackwardArgs g{(const float4 *)grad_image, grad_depthmap, (const float4 *)image, depthmap, final_weights, ends, last,
-                   last_depth, grad_vertices, grad_colors, grad_opacities};
+                   last_depth, fragments, grad_vertices, grad_colors, grad_opacities};
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
         TG_LAUNCH(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
         return check_launch("backward_tile_order_kernel");
+    }
+    if (fragments) {
+        if (max_layers > TG_MAX_SAVED_LAYERS) {
+            set_error("tg_render_backward: saved fragments need max_layers <= %d", TG_MAX_SAVED_LAYERS);
+            return TG_E_ARG;
+        }
+        const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
+        TG_LAUNCH(backward_saved_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
+        return check_launch("backward_saved_order_kernel");
     }
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads());
     const size_t lds = backward_pixel_order_lds_bytes(tl.threads);

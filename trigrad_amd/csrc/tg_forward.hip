@@ -23,6 +23,7 @@ struct ForwardOut {
     int32_t *ends;
     int32_t *last;
     float *last_depth;
+    int32_t *fragments;  // (max_layers, H, W): list positions, relative to the tile's start, in blend order; may be null
 };
 
 __device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, float last_depth) {
@@ -173,6 +174,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                         float b0, b1, b2;
                         bary_apply(r[u].m, p.px, p.py, b0, b1, b2);
                         if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
+                        if (out.fragments) out.fragments[(int64_t)s.blended * ((int64_t)a.W * a.H) + p.index] = tk.j(i0 + u) - start;
                         blend_fragment(s, r[u], b0, b1, b2);
                     }
                 }
@@ -251,7 +253,7 @@ extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, 
                                  const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
                                  int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
                                  float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
-                                 float *last_depth, void *stream) {
+                                 float *last_depth, int32_t *fragments, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
         set_error("tg_render_forward: null pointer");
@@ -263,7 +265,11 @@ extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, 
     }
     RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
-    ForwardOut o{(float4 *)image, depthmap, final_weights, ends, last, last_depth};
+    if (fragments && (!per_pixel_sort || max_layers > TG_MAX_SAVED_LAYERS)) {
+        set_error("tg_render_forward: fragments are saved only with per_pixel_sort and max_layers <= %d", TG_MAX_SAVED_LAYERS);
+        return TG_E_ARG;
+    }
+    ForwardOut o{(float4 *)image, depthmap, final_weights, ends, last, last_depth, fragments};
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads() : kTileThreads);
     const dim3 grid = tl.grid;
     const int n_threads = tl.threads;

@@ -52,15 +52,17 @@ class Renderer(Function):
             (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume) = _C.render_forward(
                 vertices, indices, colors, opacities, width, height, tile_width, tile_height, early_stopping_threshold,
                 not record_timing, per_pixel_sort, max_layers)
-            last, last_depth, sort_status = resume
+            last, last_depth, sort_status, fragments = resume
             if record_timing and int(sort_status.item()) != 0:
                 raise RuntimeError("tg_sort_pairs_u64_u32: look-back wait timed out")
+            # private to this Function: where the reverse traversal starts, and (per-pixel order,
+            # max_layers <= 32) the blend order itself
+            extras = [t for t in (last_depth, fragments) if t is not None]
             ctx.has_last_depth = last_depth is not None
+            ctx.has_fragments = fragments is not None
             saved = [vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, image, depthmap, final_weights,
                      ends, last, sort_status]
-            if last_depth is not None:
-                saved.append(last_depth)
-            ctx.save_for_backward(*saved)
+            ctx.save_for_backward(*saved, *extras)
         if record_timing:
             return image, depthmap, timings
         return image, depthmap
@@ -74,7 +76,9 @@ class Renderer(Function):
         else:
             saved = ctx.saved_tensors
             last, sort_status = saved[11], saved[12]
-            last_depth = saved[13] if ctx.has_last_depth else None
+            extras = list(saved[13:])
+            last_depth = extras.pop(0) if ctx.has_last_depth else None
+            fragments = extras.pop(0) if ctx.has_fragments else None
             width, height, tile_width, tile_height, threshold, per_pixel_sort, max_layers = ctx.render_args
             if grad_image is None:
                 grad_image = torch.zeros_like(saved[7])
@@ -82,7 +86,7 @@ class Renderer(Function):
                 grad_depthmap = torch.zeros_like(saved[8])
             grad_vertices, grad_colors, grad_opacities = _C.render_backward(
                 grad_image, grad_depthmap, *saved[:11], width, height, tile_width, tile_height, threshold, per_pixel_sort,
-                max_layers, resume=(last, last_depth, sort_status))
+                max_layers, resume=(last, last_depth, sort_status, fragments))
         # one slot per forward argument (wrapper.py:99-112)
         return (grad_vertices, None, grad_colors, grad_opacities, None, None, None, None, None, None, None, None)
 
