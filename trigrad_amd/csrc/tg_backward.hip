@@ -590,17 +590,27 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 // Per-pixel order with the blend order saved by the forward pass
 // (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  The records of the first
 // kSavedWindow list entries of the tile are staged once (rows an odd number of
-// words apart, so lanes reading different entries use different banks) and the
-// gradient sums of those entries are kept in LDS; later entries are gathered
-// from and added to memory directly.
+// words apart, so lanes reading different entries use different banks).  Every
+// wave walks its 64 pixels in lockstep, each lane from its own far end.  LDS
+// float atomics cost about three cycles per lane on gfx950 and many lanes of a
+// wave hold the same entry in the same step, so the 21 gradient terms of a step
+// are grouped by entry first: lanes with equal entries get consecutive slots
+// (ballot matching, groups in order of their lowest lane), the terms go to a
+// slot-major matrix in LDS, three groups of 21 lanes add up the runs of equal
+// entry and issue one global float atomic per run and term.  Fragments of
+// entries beyond the staged window are gathered from and added to memory
+// directly.
 constexpr int kSavedWindow = 256;
 constexpr int kBackWords = (int)(sizeof(BackRecord) / sizeof(float));  // 36
 constexpr int kSavedStride = kBackWords + 1;
 
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ float s_rows[kSavedWindow * kSavedStride];
-    __shared__ float s_acc[kSavedWindow * kTerms];
+    __shared__ float s_term[kMaxWaves][kTerms * kTermStride];
+    __shared__ int s_tag[kMaxWaves][kWave];
     const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
@@ -612,50 +622,93 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
 #pragma unroll
         for (int k = 0; k < kBackWords; k++) s_rows[e * kSavedStride + k] = w[k];
     }
-    for (int i = tid; i < n_win * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
     __syncthreads();
+    float *terms = s_term[wave];
+    int *tags = s_tag[wave];
 
+    BackState st;
+    int n = 0;
     if (p.valid) {
-        BackState st = load_back_state(g, p);
-        const int n = min(g.ends[p.index], a.max_layers);  // render.cu:642
-        const int64_t plane = (int64_t)a.W * a.H;
-        for (int hi = n; hi > 0; hi -= kGatherAhead) {
-            int rel[kGatherAhead];
+        st = load_back_state(g, p);
+        n = min(g.ends[p.index], a.max_layers);  // render.cu:642
+    }
+    int n_max = n;
 #pragma unroll
-            for (int u = 0; u < kGatherAhead; u++) rel[u] = g.fragments[(int64_t)max(hi - 1 - u, 0) * plane + p.index];
+    for (int off = 32; off > 0; off >>= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
+    const int64_t plane = (int64_t)a.W * a.H;
+    // step s of a lane is its layer n - 1 - s: every lane starts at its own far end
+    for (int s0 = 0; s0 < n_max; s0 += kGatherAhead) {
+        int rel[kGatherAhead];
 #pragma unroll
-            for (int u = 0; u < kGatherAhead; u++) {
-                if (hi - 1 - u < 0) break;
+        for (int u = 0; u < kGatherAhead; u++)
+            rel[u] = (n > 0) ? g.fragments[(int64_t)max(n - 1 - s0 - u, 0) * plane + p.index] : 0;
+#pragma unroll
+        for (int u = 0; u < kGatherAhead; u++) {
+            if (s0 + u >= n_max) break;  // wave-uniform
+            const bool active = s0 + u < n;
+            const bool staged = active && rel[u] < n_win;
+            float term[kTerms];
+            if (active) {
                 BackRecord r;
-                if (rel[u] < n_win) {
+                if (staged) {
                     float *w = reinterpret_cast<float *>(&r);
 #pragma unroll
-                    for (int k = 0; k < kBackWords; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
+                    for (int k = 0; k < kBackWords - 3; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
                 } else {
                     gather_back(a, start + rel[u], r);
                 }
                 float b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                float term[kTerms];
                 fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
-                if (rel[u] < n_win) {
-#pragma unroll
-                    for (int q = 0; q < kTerms; q++) atomicAdd(s_acc + rel[u] * kTerms + q, term[q]);
-                } else {
+                if (!staged) {
 #pragma unroll
                     for (int q = 0; q < kTerms; q++)
                         if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
                 }
             }
-        }
-    }
-    __syncthreads();
-    for (int e = tid; e < n_win; e += blockDim.x) {
-        const int *id = reinterpret_cast<const int *>(s_rows + e * kSavedStride + (kBackWords - 3));
+            // slots: lanes with the same entry next to each other, groups in order of their lowest lane
+            uint64_t peers = __builtin_amdgcn_ballot_w64(staged);
+            if (peers == 0) continue;  // wave-uniform
 #pragma unroll
-        for (int q = 0; q < kTerms; q++) {
-            const float v = s_acc[e * kTerms + q];
-            if (v != 0.0f) unsafeAtomicAdd(term_address(g, id[q / 7], q % 7), v);
+            for (int b = 0; b < 8; b++) {
+                const bool bit = (rel[u] >> b) & 1;
+                const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
+                peers &= bit ? vote : ~vote;
+            }
+            const uint32_t rank = lanes_below_mask(peers);
+            const bool leads = staged && rank == 0;
+            const uint32_t size = leads ? (uint32_t)__builtin_popcountll(peers) : 0u;
+            const uint32_t incl = wave_inclusive_scan_u32(size);
+            const int n_slots = __builtin_amdgcn_readlane((int)incl, kWave - 1);
+            const int leader = staged ? __builtin_ctzll(peers) : lane;
+            const int slot = __shfl((int)(incl - size), leader, kWave) + (int)rank;
+            if (staged) {
+#pragma unroll
+                for (int q = 0; q < kTerms; q++) terms[q * kTermStride + slot] = term[q];
+                tags[slot] = rel[u];
+            }
+            wave_lds_sync();
+            // lanes (group, q): group 0..2 owns a third of the slots; runs of equal entry are contiguous
+            const int group = lane / kTerms, q = lane - group * kTerms;
+            const int per = (n_slots + 2) / 3;
+            const int c0 = group * per, c1 = min(c0 + per, n_slots);
+            if (group < 3 && c0 < c1) {
+                int cur = tags[c0];
+                float sum = 0.0f;
+                for (int c = c0; c < c1; c++) {
+                    const int t = tags[c];
+                    if (t != cur) {
+                        if (sum != 0.0f)
+                            unsafeAtomicAdd(term_address(g, __float_as_int(s_rows[cur * kSavedStride + kBackWords - 3 + q / 7]), q % 7), sum);
+                        sum = 0.0f;
+                        cur = t;
+                    }
+                    sum += terms[q * kTermStride + c];
+                }
+                if (sum != 0.0f)
+                    unsafeAtomicAdd(term_address(g, __float_as_int(s_rows[cur * kSavedStride + kBackWords - 3 + q / 7]), q % 7), sum);
+            }
+            wave_lds_sync();
         }
     }
 }
