@@ -157,17 +157,44 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 topk_insert(tk, cap, found, pd, j);
             }
         }
+        // Selection is over: the staging area and the depth lists are dead apart from
+        // the depth of the last fragment each lane is going to blend.  The space takes
+        // the blend records of the first list entries (rows an odd number of words
+        // apart: lanes reading different entries use different banks); entries
+        // beyond it are gathered from memory.
+        const int todo = (want && found > 0) ? min(found, a.max_layers - s.blended) : 0;
+        const float todo_depth = todo > 0 ? tk.d(todo - 1) : 0.0f;
+        __syncthreads();
+        float *rows = reinterpret_cast<float *>(s_dyn);
+        const int n_rows = min(end - start, (int)((sizeof(DepthRecord) * kBatch + sizeof(float) * kLayers * n_threads) /
+                                                   (sizeof(float) * kBlendWords)));
+        for (int e = tid; e < n_rows; e += blockDim.x) {
+            BlendRecord r;
+            gather_blend(a, start + e, r);
+            const float *w = reinterpret_cast<const float *>(&r);
+#pragma unroll
+            for (int k = 0; k < kBlendWords; k++) rows[e * kBlendWords + k] = w[k];
+        }
+        __syncthreads();
         if (want) {
             if (found == 0) {
                 active = false;  // render.cu:594
             } else {
-                const int todo = min(found, a.max_layers - s.blended);
-                // kGatherAhead records are fetched together: their chains of dependent
-                // loads (list -> indices -> vertices) overlap instead of adding up
+                // kGatherAhead records are fetched together: the chains of dependent loads
+                // (list -> indices -> vertices) of those that come from memory overlap
                 for (int i0 = 0; i0 < todo; i0 += kGatherAhead) {
                     BlendRecord r[kGatherAhead];
 #pragma unroll
-                    for (int u = 0; u < kGatherAhead; u++) gather_blend(a, tk.j(min(i0 + u, todo - 1)), r[u]);
+                    for (int u = 0; u < kGatherAhead; u++) {
+                        const int rel = tk.j(min(i0 + u, todo - 1)) - start;
+                        if (rel < n_rows) {
+                            float *w = reinterpret_cast<float *>(&r[u]);
+#pragma unroll
+                            for (int k = 0; k < kBlendWords; k++) w[k] = rows[rel * kBlendWords + k];
+                        } else {
+                            gather_blend(a, start + rel, r[u]);
+                        }
+                    }
 #pragma unroll
                     for (int u = 0; u < kGatherAhead; u++) {
                         if (i0 + u >= todo) break;
@@ -178,7 +205,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                         blend_fragment(s, r[u], b0, b1, b2);
                     }
                 }
-                last_depth = tk.d(todo - 1);
+                last_depth = todo_depth;
                 last_j = tk.j(todo - 1);
                 // fewer candidates than asked for: the list is exhausted, the next
                 // selection would return nothing (render.cu:594)

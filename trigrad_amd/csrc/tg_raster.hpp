@@ -61,6 +61,7 @@ struct alignas(16) BlendRecord {
     float pad;
 };
 static_assert(sizeof(BlendRecord) == 112, "BlendRecord layout");
+constexpr int kBlendWords = 27;  // floats of a BlendRecord without its padding; odd
 
 // What select_next_k_in_tile (render.cu:375-415) reads for one list entry.
 struct alignas(16) DepthRecord {
