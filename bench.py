@@ -79,7 +79,7 @@ def main():
         verts.grad = colors.grad = opac.grad = None
         image, depthmap = trigrad_amd.render(verts, d["indices"], colors, opac, W, H, 16, 16, 1 / 256, False, **MODES[mode])
         if backward:
-            loss = ((image - d["target"]) ** 2).mean()
+            loss = torch.nn.functional.mse_loss(image, d["target"])
             loss.backward()
         return image
 

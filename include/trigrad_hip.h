@@ -151,8 +151,9 @@ int tg_render_forward(const float *vertices, const int32_t *indices, const float
 /* Accumulates into grad_vertices (V,4), grad_colors (V,3), grad_opacities (V),
  * which the caller zero-initialises.  Replaces render_backward_kernel /
  * process_backward (render.cu:455-538, 621-695).  Fragments are visited in
- * exact reverse blend order.  fragments: what tg_render_forward saved, or NULL
- * (then last and, with per_pixel_sort, last_depth locate the far end). */
+ * exact reverse blend order.  grad_depthmap may be NULL (= all zero: the depth
+ * map took no part in the loss).  fragments: what tg_render_forward saved, or
+ * NULL (then last and, with per_pixel_sort, last_depth locate the far end). */
 int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
                        const int32_t *indices, const float *colors, const float *opacities,
                        const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,

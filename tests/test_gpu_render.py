@@ -177,6 +177,30 @@ def test_render_autograd_end_to_end(cuda, oracle):
             assert_close(label, g.cpu().numpy(), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * float(np.abs(w).max()))
 
 
+def test_loss_on_depth_only(cuda, oracle):
+    """Only the depth map takes part in the loss: the image's gradient arrives as None."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import scenes as S
+    scene = S.random_soup(400, 96, 80, seed=21, sigma_px=9.0, varying_w=True)
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    v = d["vertices"].clone().requires_grad_()
+    c = d["colors"].clone().requires_grad_()
+    o = d["opacities"].clone().requires_grad_()
+    image, depthmap = trigrad_amd.render(v, d["indices"], c, o, W, H)
+    hit = torch.isfinite(depthmap)
+    weight = torch.linspace(0.5, 1.5, W * H, device=cuda).reshape(H, W)
+    (torch.where(hit, depthmap, torch.zeros_like(depthmap)) * weight).sum().backward()
+    fwd = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H)
+    gd = np.where(np.isfinite(fwd["depthmap"]), weight.cpu().numpy(), 0.0).astype(np.float32)
+    gV, gC, gO = oracle.render_backward(np.zeros((H, W, 4), np.float32), gd, scene["vertices"], scene["indices"], scene["colors"],
+                                        scene["opacities"], fwd, W, H)
+    for label, g, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
+        assert_close(label, g.cpu().numpy(), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * float(np.abs(w).max()))
+    assert float(v.grad.abs().max()) > 0
+
+
 def test_record_timing_and_empty_scene(cuda):
     import torch
     import trigrad_amd

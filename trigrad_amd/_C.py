@@ -258,7 +258,9 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
 def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
                     image, depthmap, final_weights, ends, width, height, tile_width, tile_height, early_stopping_threshold,
                     per_pixel_sort, max_layers, resume=None):
-    """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities)."""
+    """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities).
+
+    grad_depthmap may be None (no gradient reached the depth map)."""
     if resume is None:
         raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
     last, last_depth, sort_status, fragments = resume
@@ -266,11 +268,15 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
     lib = _lib.load()
     dev = vertices.device
     with torch.cuda.device(dev):
-        tensors = [t.contiguous() for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
-                                            bary_transforms, image, depthmap, final_weights, ends, last)]
-        grad_vertices = torch.zeros_like(tensors[2])
-        grad_colors = torch.zeros_like(tensors[4])
-        grad_opacities = torch.zeros_like(tensors[5])
+        tensors = [None if t is None else t.contiguous()
+                   for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
+                             bary_transforms, image, depthmap, final_weights, ends, last)]
+        # one zero fill for the three gradients: (V,4) | (V,3) | (V,) views of one block
+        V = vertices.shape[0]
+        block = torch.zeros((8 * V,), dtype=torch.float32, device=dev)
+        grad_vertices = block[:4 * V].view(V, 4)
+        grad_colors = block[4 * V:7 * V].view(V, 3)
+        grad_opacities = block[7 * V:]
         _lib.check(lib.tg_render_backward(
             *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),

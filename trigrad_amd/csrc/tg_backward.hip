@@ -250,7 +250,7 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
     BackState st;
     const float4 gi = g.grad_image[p.index];
     st.g0 = gi.x; st.g1 = gi.y; st.g2 = gi.z; st.g3 = gi.w;
-    st.gd = g.grad_depthmap[p.index];
+    st.gd = g.grad_depthmap ? g.grad_depthmap[p.index] : 0.0f;  // null: the depth map took no part in the loss
     st.final_alpha = g.image[p.index].w;
     st.alpha = st.final_alpha;
     st.s0 = st.s1 = st.s2 = 0.0f;
@@ -727,7 +727,7 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
                                   int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
                                   float *grad_colors, float *grad_opacities, void *stream) {
     if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
-    if (!grad_image || !grad_depthmap || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
+    if (!grad_image || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
         !depthmap || !final_weights || !ends || !last || !grad_vertices || !grad_colors || !grad_opacities ||
         (per_pixel_sort && !last_depth && !fragments)) {
         set_error("tg_render_backward: null pointer");

@@ -39,6 +39,7 @@ class Renderer(Function):
             max_layers = n_triangles + 1  # wrapper.py:35-36: "no limit"
 
         ctx.render_args = (width, height, tile_width, tile_height, early_stopping_threshold, per_pixel_sort, max_layers)
+        ctx.set_materialize_grads(False)  # an output the loss does not use arrives as None instead of a zero tensor
         if n_triangles < 1:
             # wrapper.py:46-53: nothing to draw -- transparent black, infinitely far
             ctx.skipped = True
@@ -82,8 +83,6 @@ class Renderer(Function):
             width, height, tile_width, tile_height, threshold, per_pixel_sort, max_layers = ctx.render_args
             if grad_image is None:
                 grad_image = torch.zeros_like(saved[7])
-            if grad_depthmap is None:
-                grad_depthmap = torch.zeros_like(saved[8])
             grad_vertices, grad_colors, grad_opacities = _C.render_backward(
                 grad_image, grad_depthmap, *saved[:11], width, height, tile_width, tile_height, threshold, per_pixel_sort,
                 max_layers, resume=(last, last_depth, sort_status, fragments))
