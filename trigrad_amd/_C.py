@@ -67,6 +67,8 @@ SAVE_BLEND_ORDER = True
 def scan_exclusive(counts, out=None, heads=None):
     """Exclusive prefix sum of an int32 tensor -> (offsets, total (1,) int32, status (1,) int32).
 
+    total and status are the two halves of one (2,) tensor (`total._base`).
+
     heads (optional int32 tensor): receives, for every multiple of OWNER_STRIDE
     below the total, the index of the element that owns that output position.
     """
@@ -75,8 +77,8 @@ def scan_exclusive(counts, out=None, heads=None):
     n = counts.numel()
     dev = counts.device
     out = torch.empty_like(counts) if out is None else out
-    total = torch.empty((1,), dtype=torch.int32, device=dev)
-    status = torch.empty((1,), dtype=torch.int32, device=dev)
+    pair = torch.empty((2,), dtype=torch.int32, device=dev)  # one allocation, so that one copy brings both to the host
+    total, status = pair[:1], pair[1:]
     ws_bytes = int(lib.tg_scan_workspace_bytes(n))
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -117,7 +119,7 @@ def sort_pairs(keys, values, end_bit=64):
     dev = keys.device
     keys_alt = torch.empty_like(keys)
     values_alt = torch.empty_like(values)
-    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    status = torch.empty((1,), dtype=torch.int32, device=dev)  # the library writes it in every path
     ws_bytes = int(lib.tg_sort_workspace_bytes(n))
     ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
     in_alt = C.c_int(0)
@@ -164,7 +166,7 @@ def per_tile_lists(vertices, indices, width, height, tile_width, tile_height):
     counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
     heads = owner_heads_for(indices.shape[0], vertices.device)
     tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
-    host = torch.stack([total[0], status[0]]).cpu()  # the one device->host read of the forward pass
+    host = total._base.cpu()  # the one device->host read of the forward pass
     K, st = int(host[0]), int(host[1])
     if st != 0:
         raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
@@ -231,7 +233,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
         heads = owner_heads_for(indices.shape[0], dev)
         tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
-        host = torch.stack([total[0], status[0]]).cpu()
+        host = total._base.cpu()
         K, st = int(host[0]), int(host[1])
         if st != 0:
             raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
