@@ -11,7 +11,7 @@
  *   - the return value is 0 on success, a negative TG_E_* code for rejected
  *     arguments, or a positive hipError_t; tg_last_error() describes the last
  *     failure on the calling thread;
- *   - data layout is the reference's: vertices (V,4) float32
+ *   - data layout is the reference's: vertices (V,4) tg_real
  *     (x/w, y/w, z/w, 1/w), indices (M,3) int32, colors (V,3), opacities (V),
  *     image (H,W,4) with remaining transmittance in channel 3, row 0 at
  *     y = -1 (reference src/trigrad/wrapper.py:131-141, render.cu:557-562).
@@ -31,16 +31,27 @@ extern "C" {
 
 #define TG_ABI_VERSION 1
 
+/* The scalar type of the build, like the reference's `scalar` (util.h:5-20):
+ * libtrigrad_hip.so is built with float, libtrigrad_hip_f64.so with
+ * -DTG_DOUBLE_PRECISION (the reference's DOUBLE_PRECISION switch, which lets
+ * its gradcheck tests run).  tg_precision_bits() tells which one a library is. */
+#ifdef TG_DOUBLE_PRECISION
+typedef double tg_real;
+#else
+typedef float tg_real;
+#endif
+
 #define TG_E_ARG (-1)       /* null pointer, negative size, unsupported tile size */
 #define TG_E_WORKSPACE (-2) /* workspace too small */
 
-/* Status word values written by the kernels that wait on other workgroups. */
 #define TG_MAX_SAVED_LAYERS 32 /* largest max_layers for which the forward pass can save the blend order */
 
+/* Status word values written by the kernels that wait on other workgroups. */
 #define TG_STATUS_OK 0u
 #define TG_STATUS_LOOKBACK_TIMEOUT 1u
 
 int tg_version(void);
+int tg_precision_bits(void); /* 32 or 64 */
 const char *tg_last_error(void);
 
 /* Number of tiles of a W x H image (reference render.cu:105-106). */
@@ -63,7 +74,7 @@ int tg_profile_report(char *buffer, size_t capacity);
  * Replaces count_per_tile / count_per_tile_kernel / touched_tiles
  * (render.cu:51-76, 90-139); the per-tile histogram of the reference is not
  * needed by the key pipeline (the tile ranges come out of the sort). */
-int tg_bin_count(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+int tg_bin_count(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
                  int tile_h, uint32_t *tri_counts, void *stream);
 
 /* Exclusive prefix sum of n uint32 (single pass, decoupled look-back).
@@ -85,12 +96,16 @@ int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t
  *   payload[pos] = i
  * where depth_key is the minimum of the triangle's z plane over the triangle
  * clipped to the tile (1e30 when the clip is empty) and orderable() is the
- * order-preserving map of float bits to uint32.  Replaces
+ * order-preserving map of tg_real bits to uint32.  Replaces
  * fill_per_tile_lists_kernel, compute_plane, clip_polygon_to_halfspace
  * (render.cu:140-270).  n_keys = total of the scan.  owner_heads (may be NULL)
  * is the scan's `heads` output for head_stride = 256 with owner_capacity
- * entries; without it the owners are found by binary search. */
-int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+ * entries; without it the owners are found by binary search.
+ * Double-precision build: a depth key needs all 64 bits, so keys holds
+ * 2 * n_keys words, keys[pos] = orderable(depth_key) and
+ * keys[n_keys + pos] = tile_id; the caller sorts by depth, then stably by tile
+ * (two calls of tg_sort_pairs_u64_u32). */
+int tg_bin_emit(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
                 int tile_h, const uint32_t *tri_offsets, int64_t n_keys, const uint32_t *owner_heads,
                 uint32_t owner_capacity, uint64_t *keys, uint32_t *payload, void *stream);
 
@@ -120,7 +135,7 @@ int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int
 /* Row-major 3x3 cartesian-to-barycentric matrix per triangle, out is (M,3,3).
  * Replaces cartesian_to_bary / cartesian_to_bary_kernel (render.cu:310-337,
  * 697-711), also exported by the reference as _C.cartesian_to_bary. */
-int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, float *out,
+int tg_bary(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, tg_real *out,
             void *stream);
 
 /* ---- (4) forward blend ------------------------------------------------------ */
@@ -140,11 +155,11 @@ int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, i
  * tg_render_backward then walks them backwards instead of selecting the
  * fragments again (the reference re-selects, render.cu:667-693).
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
-int tg_render_forward(const float *vertices, const int32_t *indices, const float *colors, const float *opacities,
-                      const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
-                      int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
-                      float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
-                      float *last_depth, int32_t *fragments, void *stream);
+int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_real *colors, const tg_real *opacities,
+                      const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, int width, int height,
+                      int tile_w, int tile_h, tg_real early_stopping_threshold, int per_pixel_sort, int max_layers,
+                      tg_real *image, tg_real *depthmap, tg_real *final_weights, int32_t *ends, int32_t *last,
+                      tg_real *last_depth, int32_t *fragments, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
 
@@ -154,13 +169,13 @@ int tg_render_forward(const float *vertices, const int32_t *indices, const float
  * exact reverse blend order.  grad_depthmap may be NULL (= all zero: the depth
  * map took no part in the loss).  fragments: what tg_render_forward saved, or
  * NULL (then last and, with per_pixel_sort, last_depth locate the far end). */
-int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
-                       const int32_t *indices, const float *colors, const float *opacities,
-                       const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
-                       const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
-                       const float *last_depth, const int32_t *fragments, int width, int height, int tile_w, int tile_h,
-                       float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
-                       float *grad_colors, float *grad_opacities, void *stream);
+int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, const tg_real *vertices,
+                       const int32_t *indices, const tg_real *colors, const tg_real *opacities,
+                       const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, const tg_real *image,
+                       const tg_real *depthmap, const tg_real *final_weights, const int32_t *ends, const int32_t *last,
+                       const tg_real *last_depth, const int32_t *fragments, int width, int height, int tile_w, int tile_h,
+                       tg_real early_stopping_threshold, int per_pixel_sort, int max_layers, tg_real *grad_vertices,
+                       tg_real *grad_colors, tg_real *grad_opacities, void *stream);
 
 /* ---- host-side component hooks ---------------------------------------------- */
 
@@ -168,17 +183,17 @@ int tg_render_backward(const float *grad_image, const float *grad_depthmap, cons
  * from its extension for its component tests (tests.cu:43-76: barycentric_torch,
  * barycentric_backward_torch, interpolate3_scalar_torch, ..._backward_torch,
  * interpolate3_vector_torch, ..._backward_torch around util.h:232-250, 299-355,
- * 395-455).  2-vectors and 3-vectors are plain float arrays. */
-void tg_barycentric(const float *v0, const float *v1, const float *v2, const float *p, float *out3);
-void tg_barycentric_backward(const float *g3, const float *a, const float *b, const float *c, const float *p,
-                             float *grads_4x2);
-float tg_interpolate3_scalar(const float *bary, float a, float b, float c, const float *w);
-void tg_interpolate3_scalar_backward(float g, const float *bary, float a, float b, float c, const float *w,
-                                     float *grad_bary, float *grad_values, float *grad_w);
-void tg_interpolate3_vector(const float *bary, const float *a, const float *b, const float *c, const float *w, float *out3);
-void tg_interpolate3_vector_backward(const float *g3, const float *bary, const float *a, const float *b, const float *c,
-                                     const float *w, float *grad_bary, float *grad_a, float *grad_b, float *grad_c,
-                                     float *grad_w);
+ * 395-455).  2-vectors and 3-vectors are plain tg_real arrays. */
+void tg_barycentric(const tg_real *v0, const tg_real *v1, const tg_real *v2, const tg_real *p, tg_real *out3);
+void tg_barycentric_backward(const tg_real *g3, const tg_real *a, const tg_real *b, const tg_real *c, const tg_real *p,
+                             tg_real *grads_4x2);
+tg_real tg_interpolate3_scalar(const tg_real *bary, tg_real a, tg_real b, tg_real c, const tg_real *w);
+void tg_interpolate3_scalar_backward(tg_real g, const tg_real *bary, tg_real a, tg_real b, tg_real c, const tg_real *w,
+                                     tg_real *grad_bary, tg_real *grad_values, tg_real *grad_w);
+void tg_interpolate3_vector(const tg_real *bary, const tg_real *a, const tg_real *b, const tg_real *c, const tg_real *w, tg_real *out3);
+void tg_interpolate3_vector_backward(const tg_real *g3, const tg_real *bary, const tg_real *a, const tg_real *b, const tg_real *c,
+                                     const tg_real *w, tg_real *grad_bary, tg_real *grad_a, tg_real *grad_b, tg_real *grad_c,
+                                     tg_real *grad_w);
 
 #ifdef __cplusplus
 }

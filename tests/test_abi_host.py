@@ -17,20 +17,24 @@ def _declared_entry_points():
     return sorted(set(re.findall(r"\b(tg_[a-z0-9_]+)\s*\(", text)))
 
 
-def test_library_exports_every_declared_entry_point():
+@pytest.mark.parametrize("bits", [32, 64])
+def test_library_exports_every_declared_entry_point(bits):
+    """Both builds of the library (float, and double = the reference's DOUBLE_PRECISION)."""
     from trigrad_amd import _lib
-    lib = _lib.load()
+    lib = _lib.load(bits)
     names = _declared_entry_points()
     assert len(names) >= 14
     for name in names:
         assert hasattr(lib, name), f"{name} is declared in include/trigrad_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "trigrad_amd/_lib.py must declare exactly the header's entry points"
     assert lib.tg_version() == 1
+    assert lib.tg_precision_bits() == bits
 
 
-def test_host_side_helpers_and_argument_rejection():
+@pytest.mark.parametrize("bits", [32, 64])
+def test_host_side_helpers_and_argument_rejection(bits):
     from trigrad_amd import _lib
-    lib = _lib.load()
+    lib = _lib.load(bits)
     assert lib.tg_num_tiles(1920, 1080, 16, 16) == 120 * 68
     assert lib.tg_num_tiles(50, 50, 4, 4) == 13 * 13
     assert lib.tg_num_tiles(0, 10, 16, 16) == 0
@@ -52,7 +56,7 @@ def test_host_side_helpers_and_argument_rejection():
     assert b"max_layers" in lib.tg_last_error()
     assert lib.tg_render_backward(*([None] * 16), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, None) == -1
     with pytest.raises(RuntimeError, match="tg_bin_count failed with code -1"):
-        _lib.check(lib.tg_bin_count(None, 0, None, -1, 64, 64, 16, 16, None, None), "tg_bin_count")
+        _lib.check(lib.tg_bin_count(None, 0, None, -1, 64, 64, 16, 16, None, None), "tg_bin_count", bits)
 
 
 def test_python_entry_point_errors_without_gpu():

@@ -12,9 +12,19 @@ import ctypes as C
 
 import torch
 
+import os
+
 from . import _lib
 
-precision = torch.float32  # module.cu:17-21; this build is the float32 one
+# The reference fixes its scalar type when the extension is compiled (util.h:5-20, module.cu:17-21).
+# Here both builds of the library are present; TRIGRAD_PRECISION=float64 (or set_precision) selects the
+# double one, which the entry points then expect, like a reference built with DOUBLE_PRECISION.
+precision = torch.float64 if os.environ.get("TRIGRAD_PRECISION", "float32").lower() in ("float64", "double", "64") else torch.float32
+
+
+def _bits(t):
+    """Which library serves tensor t: the double build for float64 data, the float build otherwise."""
+    return 64 if t.dtype == torch.float64 else 32
 
 STAGE_KEYS = ("init", "per_tile_lists", "sorting", "bary_transforms", "rasterization")  # render.cu:723-747
 
@@ -47,12 +57,12 @@ def key_bits(n_tiles):
 def bin_count(vertices, indices, width, height, tile_width, tile_height):
     """Per-triangle tile-overlap counts, (M,) int32."""
     _need_cuda(vertices, indices)
-    lib = _lib.load()
+    lib = _lib.load(_bits(vertices))
     M = indices.shape[0]
     counts = torch.empty((M,), dtype=torch.int32, device=vertices.device)
     with torch.cuda.device(vertices.device):
         _lib.check(lib.tg_bin_count(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
-                                    _ptr(counts), _stream(vertices)), "tg_bin_count")
+                                    _ptr(counts), _stream(vertices)), "tg_bin_count", _bits(vertices))
     return counts
 
 
@@ -94,16 +104,18 @@ def owner_heads_for(n_triangles, device):
 
 
 def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, tile_height, heads=None):
-    """-> (keys (K,) int64 holding uint64 bit patterns, payload (K,) int32) in emission order."""
+    """-> (keys (K,) int64 holding uint64 bit patterns, payload (K,) int32) in emission order.
+
+    float64 vertices: keys has 2K entries, the depth keys (all 64 bits) followed by the tile ids."""
     _need_cuda(vertices, indices, tri_offsets)
-    lib = _lib.load()
+    lib = _lib.load(_bits(vertices))
     dev = vertices.device
-    keys = torch.empty((n_keys,), dtype=torch.int64, device=dev)
+    keys = torch.empty((n_keys * (2 if _bits(vertices) == 64 else 1),), dtype=torch.int64, device=dev)
     payload = torch.empty((n_keys,), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(lib.tg_bin_emit(_ptr(vertices), vertices.shape[0], _ptr(indices), indices.shape[0], width, height, tile_width,
                                    tile_height, _ptr(tri_offsets), n_keys, _ptr(heads), 0 if heads is None else heads.numel(),
-                                   _ptr(keys), _ptr(payload), _stream(vertices)), "tg_bin_emit")
+                                   _ptr(keys), _ptr(payload), _stream(vertices)), "tg_bin_emit", _bits(vertices))
     return keys, payload
 
 
@@ -145,13 +157,13 @@ def tile_ranges(sorted_keys, n_tiles):
 def cartesian_to_bary(vertices, indices):
     """(M,3,3) cartesian-to-barycentric matrices (reference _C.cartesian_to_bary, render.cu:697-711)."""
     _need_cuda(vertices, indices)
-    lib = _lib.load()
+    lib = _lib.load(_bits(vertices))
     vertices = vertices.contiguous()
     indices = indices.contiguous()
     M = indices.shape[0]
-    out = torch.empty((M, 3, 3), dtype=torch.float32, device=vertices.device)
+    out = torch.empty((M, 3, 3), dtype=vertices.dtype, device=vertices.device)
     with torch.cuda.device(vertices.device):
-        _lib.check(lib.tg_bary(_ptr(vertices), vertices.shape[0], _ptr(indices), M, _ptr(out), _stream(vertices)), "tg_bary")
+        _lib.check(lib.tg_bary(_ptr(vertices), vertices.shape[0], _ptr(indices), M, _ptr(out), _stream(vertices)), "tg_bary", _bits(vertices))
     return out
 
 
@@ -170,10 +182,33 @@ def per_tile_lists(vertices, indices, width, height, tile_width, tile_height):
     K, st = int(host[0]), int(host[1])
     if st != 0:
         raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
-    keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
-    keys, payload, sort_status = sort_pairs(keys, payload, key_bits(T))
-    offsets = tile_ranges(keys, T)
+    keys, payload, sort_status, offsets = emit_and_sort(vertices, indices, tri_offsets, K, T, width, height, tile_width,
+                                                        tile_height, heads)
     return payload, offsets, keys, sort_status
+
+
+def emit_and_sort(vertices, indices, tri_offsets, K, T, width, height, tile_width, tile_height, heads):
+    """Key emission, sort and tile ranges -> (sorted_keys, sorted_ids, sort_status, offsets)."""
+    keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
+    return sort_lists(keys, payload, K, T)
+
+
+def sort_lists(keys, payload, K, T):
+    """bin_emit's output -> (sorted_keys, sorted_ids, sort_status, offsets).
+
+    float32 (K keys): one sort of (tile << 32 | depth bits).  float64 (2K keys: depth keys, then tile ids): the
+    depth takes all 64 key bits, so the pairs are sorted by depth first and then, stably, by tile id;
+    sorted_keys are then (tile << 32) only.
+    """
+    if keys.numel() == K:
+        keys, payload, sort_status = sort_pairs(keys, payload, key_bits(T))
+        return keys, payload, sort_status, tile_ranges(keys, T)
+    depth_keys, tile_ids = keys[:K], keys[K:]
+    order = torch.arange(K, dtype=torch.int32, device=keys.device)
+    _, order, status1 = sort_pairs(depth_keys, order, 64)
+    tile_keys, order, status2 = sort_pairs(tile_ids[order.long()], order, key_bits(T) - 32)
+    sorted_keys = tile_keys << 32
+    return sorted_keys, payload[order.long()], torch.maximum(status1, status2), tile_ranges(sorted_keys, T)
 
 
 class _StageTimer:
@@ -210,7 +245,9 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
     plus the sort's status word.
     """
     _need_cuda(vertices, indices, colors, opacities)
-    lib = _lib.load()
+    bits = _bits(vertices)
+    lib = _lib.load(bits)
+    real = vertices.dtype
     timer = _StageTimer(disable_timing)
     dev = vertices.device
     with torch.cuda.device(dev):
@@ -219,12 +256,12 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         indices = indices.contiguous()
         colors = colors.contiguous()
         opacities = opacities.contiguous()
-        image = torch.empty((height, width, 4), dtype=torch.float32, device=dev)
-        depthmap = torch.empty((height, width), dtype=torch.float32, device=dev)
-        final_weights = torch.empty((height, width), dtype=torch.float32, device=dev)
+        image = torch.empty((height, width, 4), dtype=real, device=dev)
+        depthmap = torch.empty((height, width), dtype=real, device=dev)
+        final_weights = torch.empty((height, width), dtype=real, device=dev)
         ends = torch.empty((height, width), dtype=torch.int32, device=dev)
         last = torch.empty((height, width), dtype=torch.int32, device=dev)
-        last_depth = torch.empty((height, width), dtype=torch.float32, device=dev) if per_pixel_sort else None
+        last_depth = torch.empty((height, width), dtype=real, device=dev) if per_pixel_sort else None
         save_order = bool(per_pixel_sort) and SAVE_BLEND_ORDER and 0 < int(max_layers) <= MAX_SAVED_LAYERS
         fragments = torch.empty((int(max_layers), height, width), dtype=torch.int32, device=dev) if save_order else None
 
@@ -240,8 +277,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
 
         timer.start("sorting")
-        keys, sorted_ids, sort_status = sort_pairs(keys, payload, key_bits(T))
-        offsets = tile_ranges(keys, T)
+        keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
 
         timer.start("bary_transforms")
         bary_transforms = cartesian_to_bary(vertices, indices)
@@ -251,7 +287,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
             width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
             _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
-            _stream(vertices)), "tg_render_forward")
+            _stream(vertices)), "tg_render_forward", bits)
         timings = timer.stop()
     return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
             (last, last_depth, sort_status, fragments))
@@ -267,7 +303,8 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
         raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
     last, last_depth, sort_status, fragments = resume
     _need_cuda(grad_output, vertices)
-    lib = _lib.load()
+    bits = _bits(vertices)
+    lib = _lib.load(bits)
     dev = vertices.device
     with torch.cuda.device(dev):
         tensors = [None if t is None else t.contiguous()
@@ -275,14 +312,14 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
                              bary_transforms, image, depthmap, final_weights, ends, last)]
         # one zero fill for the three gradients: (V,4) | (V,3) | (V,) views of one block
         V = vertices.shape[0]
-        block = torch.zeros((8 * V,), dtype=torch.float32, device=dev)
+        block = torch.zeros((8 * V,), dtype=vertices.dtype, device=dev)
         grad_vertices = block[:4 * V].view(V, 4)
         grad_colors = block[4 * V:7 * V].view(V, 3)
         grad_opacities = block[7 * V:]
         _lib.check(lib.tg_render_backward(
             *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
-            _ptr(grad_opacities), _stream(vertices)), "tg_render_backward")
+            _ptr(grad_opacities), _stream(vertices)), "tg_render_backward", bits)
     return grad_vertices, grad_colors, grad_opacities
 
 
@@ -302,3 +339,12 @@ def profile_report():
         name, count, ms = line.split()
         out[name] = (int(count), float(ms))
     return out
+
+
+def set_precision(dtype):
+    """Selects the scalar type the public entry points expect (torch.float32 or torch.float64)."""
+    global precision
+    if dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"precision must be torch.float32 or torch.float64, got {dtype}")
+    _lib.load(64 if dtype == torch.float64 else 32)
+    precision = dtype

@@ -2,8 +2,9 @@
 rasterizer behind the reference's Python entry point (`render`, `precision`)."""
 from . import camera
 from .tests_wrapper import barycentric, interpolate3_scalar, interpolate3_vector
+from ._C import set_precision
 from .wrapper import Renderer, precision, render
 
-__all__ = ["render", "barycentric", "interpolate3_scalar", "interpolate3_vector", "precision", "Renderer", "camera"]
+__all__ = ["render", "barycentric", "interpolate3_scalar", "interpolate3_vector", "precision", "Renderer", "camera", "set_precision"]
 
 __version__ = "0.1.0"

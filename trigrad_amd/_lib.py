@@ -7,19 +7,26 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# TRIGRAD_HIP_LIB names another build of the same library (same ABI), e.g. one made with different tuning constants
-LIB_PATH = os.environ.get("TRIGRAD_HIP_LIB") or os.path.join(_HERE, "lib", "libtrigrad_hip.so")
+# One library per scalar type, like the reference's compile-time DOUBLE_PRECISION switch (util.h:5-20).
+# TRIGRAD_HIP_LIB names another build of the float library (same ABI), e.g. one made with different tuning constants.
+LIB_PATHS = {
+    32: os.environ.get("TRIGRAD_HIP_LIB") or os.path.join(_HERE, "lib", "libtrigrad_hip.so"),
+    64: os.path.join(_HERE, "lib", "libtrigrad_hip_f64.so"),
+}
+LIB_PATH = LIB_PATHS[32]
 
 _p = C.c_void_p
 _i = C.c_int
 _i32 = C.c_int32
 _i64 = C.c_int64
-_f = C.c_float
 _sz = C.c_size_t
+_f = "tg_real"  # placeholder: c_float in the float library, c_double in the double one
+
 
 # name -> (restype, argtypes); the order is that of include/trigrad_hip.h
 SIGNATURES = {
     "tg_version": (_i, []),
+    "tg_precision_bits": (_i, []),
     "tg_last_error": (C.c_char_p, []),
     "tg_num_tiles": (_i, [_i, _i, _i, _i]),
     "tg_profile_enable": (None, [_i]),
@@ -42,27 +49,32 @@ SIGNATURES = {
     "tg_interpolate3_vector_backward": (None, [_p] * 11),
 }
 
-_lib = None
+_libs = {}
 
 
-def load():
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
+def load(bits=32):
+    """The library whose scalar type has `bits` bits (32: float, 64: double)."""
+    lib = _libs.get(bits)
+    if lib is None:
+        path = LIB_PATHS[bits]
+        if not os.path.exists(path):
             raise RuntimeError(
-                f"{LIB_PATH} is missing: build it with `python -m trigrad_amd.build` "
+                f"{path} is missing: build it with `python -m trigrad_amd.build` "
                 "(hipcc --offload-arch=gfx950); trigrad_amd has no other backend")
-        lib = C.CDLL(LIB_PATH)
+        lib = C.CDLL(path)
+        real = C.c_float if bits == 32 else C.c_double
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
-            fn.restype = res
-            fn.argtypes = args
-        _lib = lib
-    return _lib
+            fn.restype = real if res is _f else res
+            fn.argtypes = [real if a is _f else a for a in args]
+        if lib.tg_precision_bits() != bits:
+            raise RuntimeError(f"{path} is built for {lib.tg_precision_bits()}-bit scalars, expected {bits}")
+        _libs[bits] = lib
+    return lib
 
 
-def check(code, what):
+def check(code, what, bits=32):
     """Raise RuntimeError for a non-zero return code of an entry point."""
     if code != 0:
-        msg = load().tg_last_error()
+        msg = load(bits).tg_last_error()
         raise RuntimeError(f"{what} failed with code {code}: {msg.decode() if msg else ''}")

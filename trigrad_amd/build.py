@@ -16,6 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtrigrad_hip.so")
+LIB_PATH_F64 = os.path.join(LIB_DIR, "libtrigrad_hip_f64.so")  # the same sources with -DTG_DOUBLE_PRECISION
 
 SOURCES = ["tg_api.hip", "tg_binning.hip", "tg_scan.hip", "tg_sort.hip", "tg_forward.hip", "tg_backward.hip",
            "tg_components.hip"]
@@ -29,10 +30,9 @@ FLAGS = [
 ]
 
 
-def build(verbose=False, extra_flags=()):
-    os.makedirs(LIB_DIR, exist_ok=True)
+def _compile(out, flags, verbose):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+    cmd = [hipcc, *FLAGS, *flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", out]
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -42,6 +42,15 @@ def build(verbose=False, extra_flags=()):
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    return out
+
+
+def build(verbose=False, extra_flags=(), double_too=True):
+    """Builds the float library and (double_too) the double one; returns the float library's path."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _compile(LIB_PATH, list(extra_flags), verbose)
+    if double_too:
+        _compile(LIB_PATH_F64, [*extra_flags, "-DTG_DOUBLE_PRECISION"], verbose)
     return LIB_PATH
 
 

@@ -60,6 +60,8 @@ ProfileScope::~ProfileScope() {
 
 extern "C" int tg_version(void) { return TG_ABI_VERSION; }
 
+extern "C" int tg_precision_bits(void) { return (int)(8 * sizeof(tg_real)); }
+
 extern "C" const char *tg_last_error(void) { return tg::g_error; }
 
 extern "C" int tg_num_tiles(int width, int height, int tile_w, int tile_h) {

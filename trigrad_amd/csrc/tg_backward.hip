@@ -9,7 +9,7 @@
 //   gradient terms (3 vertices x {x, y, w, r, g, b, opacity}; the z gradient is
 //   identically zero, render.cu:531-533).  They are summed per list entry in
 //   LDS (wave-level DPP reduction when many lanes of a wave hit the same entry,
-//   LDS float atomics otherwise) and flushed with at most 21 global float
+//   LDS real atomics otherwise) and flushed with at most 21 global real
 //   atomics per (tile, entry) instead of 24 per (pixel, entry).
 // per_pixel_sort = 1: every pixel has its own order; the pixel re-selects its
 //   fragments from the far end (32 at a time, below the (depth, position) of the
@@ -20,38 +20,39 @@
 namespace tg {
 
 struct BackwardArgs {
-    const float4 *grad_image;
-    const float *grad_depthmap;
-    const float4 *image;
-    const float *depthmap;
-    const float *weights;
+    const real4 *grad_image;
+    const real *grad_depthmap;
+    const real4 *image;
+    const real *depthmap;
+    const real *weights;
     const int32_t *ends;
     const int32_t *last;
-    const float *last_depth;
+    const real *last_depth;
     const int32_t *fragments;  // saved by the forward pass, or null
-    float *grad_vertices;
-    float *grad_colors;
-    float *grad_opacities;
+    real *grad_vertices;
+    real *grad_colors;
+    real *grad_opacities;
 };
 
 // process_backward's inputs for one list entry.
 struct alignas(16) BackRecord {
-    float m[9];
-    float w[3];
-    float iw[3];
-    float op[3];
-    float col[9];
-    float xy[6];  // ax, ay, bx, by, cx, cy
+    real m[9];
+    real w[3];
+    real iw[3];
+    real op[3];
+    real col[9];
+    real xy[6];  // ax, ay, bx, by, cx, cy
     int id[3];
 };
-static_assert(sizeof(BackRecord) == 144, "BackRecord layout");
+constexpr int kBackReals = 33;  // scalars in front of the ids
+static_assert(offsetof(BackRecord, id) == kBackReals * sizeof(real), "BackRecord layout");
 
 __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackRecord &r) {
     const TriIds t = load_ids(a, j);
-    const float *m = a.bary + 9 * (int64_t)t.tri;
+    const real *m = a.bary + 9 * (int64_t)t.tri;
 #pragma unroll
     for (int k = 0; k < 9; k++) r.m[k] = m[k];
-    const float4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
+    const real4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
     r.iw[0] = 1.0f / va.w; r.iw[1] = 1.0f / vb.w; r.iw[2] = 1.0f / vc.w;
     r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
@@ -67,23 +68,23 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
 
 // Reverse-traversal state of one pixel (render.cu:647-653).
 struct BackState {
-    float final_alpha, alpha, s0, s1, s2, oa, zoa, final_weight, final_depth;
-    float g0, g1, g2, g3, gd;  // upstream gradient of this pixel
+    real final_alpha, alpha, s0, s1, s2, oa, zoa, final_weight, final_depth;
+    real g0, g1, g2, g3, gd;  // upstream gradient of this pixel
 };
 
 constexpr int kTerms = 21;  // per vertex v: [7v+0] x, [7v+1] y, [7v+2] w, [7v+3..5] rgb, [7v+6] opacity
 
 // util.h:299-317 scalar interpolate3_backward.
-__device__ __forceinline__ void interp_backward_scalar(float g, const float b[3], const float v[3], const float w[3],
-                                                       float gb[3], float gv[3], float gw[3]) {
-    const float nom = (b[0] * w[0] * v[0] + b[1] * w[1] * v[1]) + b[2] * w[2] * v[2];
-    const float denom = (b[0] * w[0] + b[1] * w[1]) + b[2] * w[2];
+__device__ __forceinline__ void interp_backward_scalar(real g, const real b[3], const real v[3], const real w[3],
+                                                       real gb[3], real gv[3], real gw[3]) {
+    const real nom = (b[0] * w[0] * v[0] + b[1] * w[1] * v[1]) + b[2] * w[2] * v[2];
+    const real denom = (b[0] * w[0] + b[1] * w[1]) + b[2] * w[2];
     if (denom * denom < kEffZero) {
 #pragma unroll
         for (int k = 0; k < 3; k++) gb[k] = gv[k] = gw[k] = 0.0f;
         return;
     }
-    const float inv2 = 1.0f / (denom * denom);
+    const real inv2 = 1.0f / (denom * denom);
 #pragma unroll
     for (int k = 0; k < 3; k++) {
         gb[k] = g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
@@ -101,40 +102,40 @@ __device__ __forceinline__ void interp_backward_scalar(float g, const float b[3]
 
 // What the ordered part hands over for one fragment.
 struct FragSeed {
-    float d_do;    // derivative w.r.t. the interpolated opacity (:502)
-    float gc[3];   // derivative w.r.t. the interpolated colour (:510)
-    float dd_dz;   // derivative w.r.t. the interpolated view depth (:517)
+    real d_do;    // derivative w.r.t. the interpolated opacity (:502)
+    real gc[3];   // derivative w.r.t. the interpolated colour (:510)
+    real dd_dz;   // derivative w.r.t. the interpolated view depth (:517)
 };
 
-__device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, float b0, float b1, float b2) {
-    const float w[3] = {r.w[0], r.w[1], r.w[2]};
-    float o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
+__device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, real b0, real b1, real b2) {
+    const real w[3] = {r.w[0], r.w[1], r.w[2]};
+    real o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
     o = clampf(o, 0.0f, kMaxOpacity);
-    float color[3];
+    real color[3];
 #pragma unroll
     for (int k = 0; k < 3; k++) color[k] = interp_w(b0, b1, b2, r.col[k], r.col[3 + k], r.col[6 + k], w[0], w[1], w[2]);
-    const float z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+    const real z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
 
-    const float om = 1.0f - o;
-    const float g[3] = {st.g0, st.g1, st.g2};
-    float s[3] = {st.s0, st.s1, st.s2};
-    float t3[3];
+    const real om = 1.0f - o;
+    const real g[3] = {st.g0, st.g1, st.g2};
+    real s[3] = {st.s0, st.s1, st.s2};
+    real t3[3];
 #pragma unroll
     for (int k = 0; k < 3; k++) t3[k] = (color[k] * st.alpha - s[k]) / om * g[k];
-    const float drgb_do = ((t3[0] + t3[1]) + t3[2]) + st.g3 * (-st.final_alpha / om);  // :491
+    const real drgb_do = ((t3[0] + t3[1]) + t3[2]) + st.g3 * (-st.final_alpha / om);  // :491
     st.alpha /= om;                                                                    // :492
 #pragma unroll
     for (int k = 0; k < 3; k++) s[k] += color[k] * o * st.alpha;                       // :493
     st.s0 = s[0]; st.s1 = s[1]; st.s2 = s[2];
-    const float ddw_do = st.alpha - st.oa / om;                                        // :494
-    const float dud_do = st.alpha * z - st.zoa / om;                                   // :495
+    const real ddw_do = st.alpha - st.oa / om;                                        // :494
+    const real dud_do = st.alpha * z - st.zoa / om;                                   // :495
     st.oa = st.oa + o * st.alpha;                                                      // :496
     st.zoa = st.zoa + z * o * st.alpha;                                                // :497
-    float dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
+    real dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
     if (st.final_weight < kEffZero) dd_do = 0.0f;
     FragSeed f;
     f.d_do = drgb_do + dd_do;
-    const float ao = st.alpha * o;
+    const real ao = st.alpha * o;
     f.gc[0] = ao * g[0]; f.gc[1] = ao * g[1]; f.gc[2] = ao * g[2];                     // :510
     f.dd_dz = ao * st.gd / st.final_weight;                                            // :517
     if (st.final_weight < kEffZero) f.dd_dz = 0.0f;
@@ -142,30 +143,30 @@ __device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const Bac
 }
 
 // The order-free part: the 21 gradient terms of one fragment.
-__device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackRecord &r, float b0, float b1, float b2, float px,
-                                               float py, float out[kTerms]) {
-    const float b[3] = {b0, b1, b2};
-    const float w[3] = {r.w[0], r.w[1], r.w[2]};
-    const float ones[3] = {1.0f, 1.0f, 1.0f};
-    float gb_o[3], gv_o[3], gw_o[3];
+__device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackRecord &r, real b0, real b1, real b2, real px,
+                                               real py, real out[kTerms]) {
+    const real b[3] = {b0, b1, b2};
+    const real w[3] = {r.w[0], r.w[1], r.w[2]};
+    const real ones[3] = {1.0f, 1.0f, 1.0f};
+    real gb_o[3], gv_o[3], gw_o[3];
     interp_backward_scalar(f.d_do, b, r.op, w, gb_o, gv_o, gw_o);
 
     // vector interpolate3_backward for the colour (util.h:319-355)
-    const float *gc = f.gc;
-    float gb_c[3] = {0.f, 0.f, 0.f}, gw_c[3] = {0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f};
+    const real *gc = f.gc;
+    real gb_c[3] = {0.f, 0.f, 0.f}, gw_c[3] = {0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f};
     {
-        float nom[3];
+        real nom[3];
 #pragma unroll
         for (int k = 0; k < 3; k++) nom[k] = (b[0] * w[0] * r.col[k] + b[1] * w[1] * r.col[3 + k]) + b[2] * w[2] * r.col[6 + k];
-        const float denom = b[0] * w[0] + b[1] * w[1] + b[2] * w[2];
+        const real denom = b[0] * w[0] + b[1] * w[1] + b[2] * w[2];
         if (!(denom * denom < kEffZero)) {
-            const float inv2 = 1.0f / (denom * denom);
+            const real inv2 = 1.0f / (denom * denom);
 #pragma unroll
             for (int v = 0; v < 3; v++) {
-                float dfb[3], dfw[3];
+                real dfb[3], dfw[3];
 #pragma unroll
                 for (int k = 0; k < 3; k++) {
-                    const float a = r.col[3 * v + k];
+                    const real a = r.col[3 * v + k];
                     dfb[k] = w[v] * (a * denom - nom[k]) * inv2;
                     dfw[k] = (b[v] * a * denom - nom[k] * b[v]) * inv2;
                 }
@@ -176,24 +177,24 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
         }
     }
 
-    float gb_z[3], gv_z[3], gw_z[3];
+    real gb_z[3], gv_z[3], gw_z[3];
     interp_backward_scalar(f.dd_dz, b, r.iw, ones, gb_z, gv_z, gw_z);
 
-    float gbary[3];
+    real gbary[3];
 #pragma unroll
     for (int k = 0; k < 3; k++) gbary[k] = gb_o[k] + gb_c[k] + gb_z[k];  // :527
 
     // util.h:405-455 barycentric_backward (vertex part)
-    const float ax = r.xy[0], ay = r.xy[1], bx = r.xy[2], by = r.xy[3], cx = r.xy[4], cy = r.xy[5];
-    float dxy[3][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    const real ax = r.xy[0], ay = r.xy[1], bx = r.xy[2], by = r.xy[3], cx = r.xy[4], cy = r.xy[5];
+    real dxy[3][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
     {
-        const float T = (bx - ax) * (cy - ay) - (by - ay) * (cx - ax);
-        const float l0 = ((bx - px) * (cy - py) - (by - py) * (cx - px)) / T;
-        const float l1 = ((cx - px) * (ay - py) - (cy - py) * (ax - px)) / T;
-        const float l2 = ((ax - px) * (by - py) - (ay - py) * (bx - px)) / T;
-        const float d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
-        if (!(fabsf(d) < kEffZero)) {
-            float J[3][2][3];
+        const real T = (bx - ax) * (cy - ay) - (by - ay) * (cx - ax);
+        const real l0 = ((bx - px) * (cy - py) - (by - py) * (cx - px)) / T;
+        const real l1 = ((cx - px) * (ay - py) - (cy - py) * (ax - px)) / T;
+        const real l2 = ((ax - px) * (by - py) - (ay - py) * (bx - px)) / T;
+        const real d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
+        if (!(abs_real(d) < kEffZero)) {
+            real J[3][2][3];
             J[0][0][0] = l0 * (-by + cy) / d;
             J[0][0][1] = (-cy - l1 * (by - cy) + py) / d;
             J[0][0][2] = (by - l2 * (by - cy) - py) / d;
@@ -220,8 +221,8 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
     }
 #pragma unroll
     for (int v = 0; v < 3; v++) {
-        const float dd_dw = -gv_z[v] / (w[v] * w[v]);   // :523-525
-        const float dw = gw_o[v] + gw_c[v] + gw_z[v];   // :530
+        const real dd_dw = -gv_z[v] / (w[v] * w[v]);   // :523-525
+        const real dw = gw_o[v] + gw_c[v] + gw_z[v];   // :530
         out[7 * v + 0] = dxy[v][0];
         out[7 * v + 1] = dxy[v][1];
         out[7 * v + 2] = dw + dd_dw;
@@ -233,13 +234,13 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
 }
 
 // One fragment start to finish (used where every pixel has its own order).
-__device__ __forceinline__ void fragment_backward(BackState &st, const BackRecord &r, float b0, float b1, float b2, float px,
-                                                  float py, float out[kTerms]) {
+__device__ __forceinline__ void fragment_backward(BackState &st, const BackRecord &r, real b0, real b1, real b2, real px,
+                                                  real py, real out[kTerms]) {
     const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
     fragment_terms(f, r, b0, b1, b2, px, py, out);
 }
 
-__device__ __forceinline__ float *term_address(const BackwardArgs &g, int vertex_id, int c) {
+__device__ __forceinline__ real *term_address(const BackwardArgs &g, int vertex_id, int c) {
     if (c < 2) return g.grad_vertices + 4 * (int64_t)vertex_id + c;
     if (c == 2) return g.grad_vertices + 4 * (int64_t)vertex_id + 3;
     if (c < 6) return g.grad_colors + 3 * (int64_t)vertex_id + (c - 3);
@@ -248,7 +249,7 @@ __device__ __forceinline__ float *term_address(const BackwardArgs &g, int vertex
 
 __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, const PixelCoord &p) {
     BackState st;
-    const float4 gi = g.grad_image[p.index];
+    const real4 gi = g.grad_image[p.index];
     st.g0 = gi.x; st.g1 = gi.y; st.g2 = gi.z; st.g3 = gi.w;
     st.gd = g.grad_depthmap ? g.grad_depthmap[p.index] : 0.0f;  // null: the depth map took no part in the loss
     st.final_alpha = g.image[p.index].w;
@@ -281,7 +282,7 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Tile-order backward.  LDS float atomics cost about three cycles per lane on
+// Tile-order backward.  LDS real atomics cost about three cycles per lane on
 // gfx950 and direct global atomics collide on the shared vertices, so the
 // per-entry sums are formed with plain LDS stores and loads.  The records of
 // 128 list entries are staged per batch by the whole workgroup; after that
@@ -299,14 +300,14 @@ __device__ __forceinline__ void wave_lds_sync() {
 //   4. order-free part, 64 slots at a time with every lane busy: lane = slot
 //      evaluates the 21 gradient terms of its hit and writes them to a term
 //      matrix; three groups of 21 lanes add up the runs of equal entry and issue
-//      one global float atomic per run and term.
+//      one global real atomic per run and term.
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ BackRecord s_rec[kBackBatch];
     __shared__ uint64_t s_ballot[kMaxWaves][kBackBatch];
     __shared__ uint32_t s_base[kMaxWaves][kBackBatch];
-    __shared__ float s_seed[kMaxWaves][kSeedWords][kWaveSlots];
-    __shared__ float s_term[kMaxWaves][kTerms * kTermStride];
-    __shared__ float s_px[kTileThreads], s_py[kTileThreads];
+    __shared__ real s_seed[kMaxWaves][kSeedWords][kWaveSlots];
+    __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
+    __shared__ real s_px[kTileThreads], s_py[kTileThreads];
     __shared__ uint8_t s_touch[kBackBatch];
     __shared__ WaveRect s_rects[kMaxTileWaves];
     __shared__ int s_last;
@@ -319,8 +320,8 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     const PixelCoord p = pixel_of_thread(a);
     uint64_t *ballots = s_ballot[wave];
     uint32_t *bases = s_base[wave];
-    float (*seeds)[kWaveSlots] = s_seed[wave];
-    float *terms = s_term[wave];
+    real (*seeds)[kWaveSlots] = s_seed[wave];
+    real *terms = s_term[wave];
 
     if (tid == 0) s_last = 0;
     s_px[tid] = p.px;
@@ -360,7 +361,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 const int bit = __builtin_ctzll(todo);
                 todo &= todo - 1;
                 const BackRecord &r = s_rec[64 * wd + bit];
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 const bool hit = bary_inside(b0, b1, b2) && 64 * wd + bit < mine;
                 const uint64_t vote = __builtin_amdgcn_ballot_w64(hit);
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 if (active) {
                     if (e >= 64) m[1] &= ~(1ull << (e - 64)); else m[0] &= ~(1ull << e);
                     const BackRecord &r = s_rec[e];
-                    float b0, b1, b2;
+                    real b0, b1, b2;
                     bary_apply(r.m, p.px, p.py, b0, b1, b2);
                     const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
                     seeds[0][slot] = f.d_do;
@@ -410,7 +411,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                     seeds[2][slot] = f.gc[1];
                     seeds[3][slot] = f.gc[2];
                     seeds[4][slot] = f.dd_dz;
-                    seeds[5][slot] = __int_as_float(e | (lane << 8));
+                    seeds[5][slot] = int_in_real(e | (lane << 8));
                 }
             }
             wave_lds_sync();
@@ -428,14 +429,14 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                     f.gc[1] = seeds[2][slot];
                     f.gc[2] = seeds[3][slot];
                     f.dd_dz = seeds[4][slot];
-                    const int packed = __float_as_int(seeds[5][slot]);
+                    const int packed = int_of_real(seeds[5][slot]);
                     tag = packed & 0xff;
                     const int src = wave * kWave + (packed >> 8);
-                    const float px = s_px[src], py = s_py[src];
+                    const real px = s_px[src], py = s_py[src];
                     const BackRecord &r = s_rec[tag];
-                    float b0, b1, b2;
+                    real b0, b1, b2;
                     bary_apply(r.m, px, py, b0, b1, b2);
-                    float term[kTerms];
+                    real term[kTerms];
                     fragment_terms(f, r, b0, b1, b2, px, py, term);
 #pragma unroll
                     for (int q = 0; q < kTerms; q++) terms[q * kTermStride + lane] = term[q];
@@ -446,10 +447,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 const int per = (n_here + 2) / 3;
                 const int c0 = group * per, c1 = min(c0 + per, n_here);
                 if (group < 3 && c0 < c1) {
-                    int cur = __float_as_int(seeds[5][s0 + c0]) & 0xff;
-                    float acc = 0.0f;
+                    int cur = int_of_real(seeds[5][s0 + c0]) & 0xff;
+                    real acc = 0.0f;
                     for (int c = c0; c < c1; c++) {
-                        const int t = __float_as_int(seeds[5][s0 + c]) & 0xff;
+                        const int t = int_of_real(seeds[5][s0 + c]) & 0xff;
                         if (t != cur) {
                             if (acc != 0.0f) unsafeAtomicAdd(term_address(g, s_rec[cur].id[q / 7], q % 7), acc);
                             acc = 0.0f;
@@ -465,13 +466,15 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     }
 }
 
-constexpr int kAccWindow = 512;  // list positions whose gradient sums are kept in LDS by the per-pixel-order kernel
+// list positions whose gradient sums are kept in LDS by the per-pixel-order kernel (the double build has
+// half the room per scalar and twice the candidate lists)
+constexpr int kAccWindow = sizeof(real) == 4 ? 512 : 128;
 
 // Candidate insertion for the reverse selection: keeps the `cap` LARGEST
 // (depth, position) pairs in descending order.  Positions arrive in ascending
 // order, so a candidate whose depth equals a stored one has the larger position
 // and goes in front of it.
-__device__ __forceinline__ void topk_insert_desc(const TopK &tk, int cap, int &n, float d, int j) {
+__device__ __forceinline__ void topk_insert_desc(const TopK &tk, int cap, int &n, real d, int j) {
     if (n == cap && d < tk.d(cap - 1)) return;
     int i = (n < cap) ? n : cap - 1;
     while (i > 0 && d >= tk.d(i - 1)) {
@@ -489,12 +492,12 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     const int n_threads = blockDim.x;
     DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
     TopK tk;
-    tk.depth = reinterpret_cast<float *>(s_dyn + sizeof(DepthRecord) * kBatch);
+    tk.depth = reinterpret_cast<real *>(s_dyn + sizeof(DepthRecord) * kBatch);
     tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
     // Per-entry sums of the first kAccWindow list positions live in LDS and are
     // flushed once per tile; positions beyond the window go straight to memory.
-    float *s_acc = reinterpret_cast<float *>(tk.pos + kLayers * n_threads);
+    real *s_acc = reinterpret_cast<real *>(tk.pos + kLayers * n_threads);
 
     __shared__ uint8_t s_touch[kBatch];
     __shared__ WaveRect s_rects[kMaxTileWaves];
@@ -511,7 +514,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     BackState st;
     int remaining = 0;
     // exclusive upper bound of the fragments still to visit, in (depth, position) order
-    float bound_depth = 0.0f;
+    real bound_depth = 0.0f;
     int bound_j = 0;
     if (p.valid) {
         st = load_back_state(g, p);
@@ -540,9 +543,9 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
                 if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
                 if (e < 0) continue;
                 const DepthRecord &r = s_rec[e];
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
+                const real pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
                 const int j = batch + e;
                 if (pd < bound_depth || (pd == bound_depth && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
             }
@@ -551,10 +554,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
             for (int i = 0; i < found; i++) {
                 BackRecord r;
                 gather_back(a, tk.j(i), r);
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
-                float term[kTerms];
+                real term[kTerms];
                 fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
                 const int rel = tk.j(i) - start;
                 if (rel < kAccWindow) {
@@ -581,7 +584,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
         const int id[3] = {t.ia, t.ib, t.ic};
 #pragma unroll
         for (int q = 0; q < kTerms; q++) {
-            const float v = s_acc[e * kTerms + q];
+            const real v = s_acc[e * kTerms + q];
             if (v != 0.0f) unsafeAtomicAdd(term_address(g, id[q / 7], q % 7), v);
         }
     }
@@ -592,21 +595,20 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 // kSavedWindow list entries of the tile are staged once (rows an odd number of
 // words apart, so lanes reading different entries use different banks).  Every
 // wave walks its 64 pixels in lockstep, each lane from its own far end.  LDS
-// float atomics cost about three cycles per lane on gfx950 and many lanes of a
+// real atomics cost about three cycles per lane on gfx950 and many lanes of a
 // wave hold the same entry in the same step, so the 21 gradient terms of a step
 // are grouped by entry first: lanes with equal entries get consecutive slots
 // (ballot matching, groups in order of their lowest lane), the terms go to a
 // slot-major matrix in LDS, three groups of 21 lanes add up the runs of equal
-// entry and issue one global float atomic per run and term.  Fragments of
+// entry and issue one global real atomic per run and term.  Fragments of
 // entries beyond the staged window are gathered from and added to memory
 // directly.
 constexpr int kSavedWindow = 256;
-constexpr int kBackWords = (int)(sizeof(BackRecord) / sizeof(float));  // 36
-constexpr int kSavedStride = kBackWords + 1;
+constexpr int kSavedStride = kBackReals + 4;  // 33 scalars, 3 vertex ids; odd
 
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
-    __shared__ float s_rows[kSavedWindow * kSavedStride];
-    __shared__ float s_term[kMaxWaves][kTerms * kTermStride];
+    __shared__ real s_rows[kSavedWindow * kSavedStride];
+    __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
     __shared__ int s_tag[kMaxWaves][kWave];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -618,12 +620,14 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     for (int e = tid; e < n_win; e += blockDim.x) {
         BackRecord r;
         gather_back(a, start + e, r);
-        const float *w = reinterpret_cast<const float *>(&r);
+        const real *w = reinterpret_cast<const real *>(&r);
 #pragma unroll
-        for (int k = 0; k < kBackWords; k++) s_rows[e * kSavedStride + k] = w[k];
+        for (int k = 0; k < kBackReals; k++) s_rows[e * kSavedStride + k] = w[k];
+#pragma unroll
+        for (int k = 0; k < 3; k++) s_rows[e * kSavedStride + kBackReals + k] = int_in_real(r.id[k]);
     }
     __syncthreads();
-    float *terms = s_term[wave];
+    real *terms = s_term[wave];
     int *tags = s_tag[wave];
 
     BackState st;
@@ -647,17 +651,17 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
             if (s0 + u >= n_max) break;  // wave-uniform
             const bool active = s0 + u < n;
             const bool staged = active && rel[u] < n_win;
-            float term[kTerms];
+            real term[kTerms];
             if (active) {
                 BackRecord r;
                 if (staged) {
-                    float *w = reinterpret_cast<float *>(&r);
+                    real *w = reinterpret_cast<real *>(&r);
 #pragma unroll
-                    for (int k = 0; k < kBackWords - 3; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
+                    for (int k = 0; k < kBackReals; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
                 } else {
                     gather_back(a, start + rel[u], r);
                 }
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
                 if (!staged) {
@@ -694,38 +698,38 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
             const int c0 = group * per, c1 = min(c0 + per, n_slots);
             if (group < 3 && c0 < c1) {
                 int cur = tags[c0];
-                float sum = 0.0f;
+                real sum = 0.0f;
                 for (int c = c0; c < c1; c++) {
                     const int t = tags[c];
                     if (t != cur) {
                         if (sum != 0.0f)
-                            unsafeAtomicAdd(term_address(g, __float_as_int(s_rows[cur * kSavedStride + kBackWords - 3 + q / 7]), q % 7), sum);
+                            unsafeAtomicAdd(term_address(g, int_of_real(s_rows[cur * kSavedStride + kBackReals + q / 7]), q % 7), sum);
                         sum = 0.0f;
                         cur = t;
                     }
                     sum += terms[q * kTermStride + c];
                 }
                 if (sum != 0.0f)
-                    unsafeAtomicAdd(term_address(g, __float_as_int(s_rows[cur * kSavedStride + kBackWords - 3 + q / 7]), q % 7), sum);
+                    unsafeAtomicAdd(term_address(g, int_of_real(s_rows[cur * kSavedStride + kBackReals + q / 7]), q % 7), sum);
             }
             wave_lds_sync();
         }
     }
 }
 
-size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads) + (size_t)kAccWindow * kTerms * sizeof(float); }
+size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads) + (size_t)kAccWindow * kTerms * sizeof(real); }
 
 }  // namespace tg
 
 using namespace tg;
 
-extern "C" int tg_render_backward(const float *grad_image, const float *grad_depthmap, const float *vertices,
-                                  const int32_t *indices, const float *colors, const float *opacities,
-                                  const int32_t *sorted_ids, const int32_t *offsets, const float *bary, const float *image,
-                                  const float *depthmap, const float *final_weights, const int32_t *ends, const int32_t *last,
-                                  const float *last_depth, const int32_t *fragments, int width, int height, int tile_w,
-                                  int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers, float *grad_vertices,
-                                  float *grad_colors, float *grad_opacities, void *stream) {
+extern "C" int tg_render_backward(const real *grad_image, const real *grad_depthmap, const real *vertices,
+                                  const int32_t *indices, const real *colors, const real *opacities,
+                                  const int32_t *sorted_ids, const int32_t *offsets, const real *bary, const real *image,
+                                  const real *depthmap, const real *final_weights, const int32_t *ends, const int32_t *last,
+                                  const real *last_depth, const int32_t *fragments, int width, int height, int tile_w,
+                                  int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers, real *grad_vertices,
+                                  real *grad_colors, real *grad_opacities, void *stream) {
     if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!grad_image || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
         !depthmap || !final_weights || !ends || !last || !grad_vertices || !grad_colors || !grad_opacities ||
@@ -737,9 +741,9 @@ extern "C" int tg_render_backward(const float *grad_image, const float *grad_dep
         set_error("tg_render_backward: vertices, image and grad_image must be 16-byte aligned");
         return TG_E_ARG;
     }
-    RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+    RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
-    BackwardArgs g{(const float4 *)grad_image, grad_depthmap, (const float4 *)image, depthmap, final_weights, ends, last,
+    BackwardArgs g{(const real4 *)grad_image, grad_depthmap, (const real4 *)image, depthmap, final_weights, ends, last,
                    last_depth, fragments, grad_vertices, grad_colors, grad_opacities};
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {

@@ -14,24 +14,24 @@ namespace tg {
 
 constexpr int kBinThreads = 256;
 
-struct TriXYZ { float ax, ay, az, bx, by, bz, cx, cy, cz; bool ok; };
+struct TriXYZ { real ax, ay, az, bx, by, bz, cx, cy, cz; bool ok; };
 
 // A triangle that names a vertex outside [0, n_vertices) is treated as
 // degenerate (all coordinates zero) instead of being dereferenced.
-__device__ __forceinline__ TriXYZ load_triangle(const float4 *__restrict__ vertices, int n_vertices,
+__device__ __forceinline__ TriXYZ load_triangle(const real4 *__restrict__ vertices, int n_vertices,
                                                 const int32_t *__restrict__ indices, int t) {
     const int ia = indices[3 * (int64_t)t], ib = indices[3 * (int64_t)t + 1], ic = indices[3 * (int64_t)t + 2];
     TriXYZ r;
     r.ok = (unsigned)ia < (unsigned)n_vertices && (unsigned)ib < (unsigned)n_vertices && (unsigned)ic < (unsigned)n_vertices;
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float4 a = r.ok ? vertices[ia] : zero, b = r.ok ? vertices[ib] : zero, c = r.ok ? vertices[ic] : zero;
+    const real4 zero = make_real4(0.f, 0.f, 0.f, 0.f);
+    const real4 a = r.ok ? vertices[ia] : zero, b = r.ok ? vertices[ib] : zero, c = r.ok ? vertices[ic] : zero;
     r.ax = a.x; r.ay = a.y; r.az = a.z;
     r.bx = b.x; r.by = b.y; r.bz = b.z;
     r.cx = c.x; r.cy = c.y; r.cz = c.z;
     return r;
 }
 
-__global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const float4 *__restrict__ vertices, int n_vertices,
+__global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                                 const int32_t *__restrict__ indices, int n_triangles, int W,
                                                                 int H, int tw, int th, int tiles_x, int tiles_y,
                                                                 uint32_t *__restrict__ tri_counts) {
@@ -46,33 +46,33 @@ __global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const float4 *__
 constexpr int kPolyCap = 8;
 constexpr int kOwnerWindow = 1024;  // triangle offsets staged per workgroup for the owner search
 struct PolyLds {
-    float x[2][kPolyCap][kBinThreads];
-    float y[2][kPolyCap][kBinThreads];
+    real x[2][kPolyCap][kBinThreads];
+    real y[2][kPolyCap][kBinThreads];
 };
 
 // One Sutherland-Hodgman pass (render.cu:159-189) from buffer `src` to `1-src`
 // against nx*x + ny*y - d >= 0.  Returns the new vertex count.  When every
 // vertex is inside, the pass reproduces its input; `src` then stays current
 // (signalled by leaving it unchanged) and no vertex is copied.
-__device__ __forceinline__ int clip_pass(PolyLds &lds, int &src, int n_in, float nx, float ny, float d) {
+__device__ __forceinline__ int clip_pass(PolyLds &lds, int &src, int n_in, real nx, real ny, real d) {
     const int tid = threadIdx.x;
     bool all_in = true;
     for (int i = 0; i < n_in; i++) all_in = all_in && (nx * lds.x[src][i][tid] + ny * lds.y[src][i][tid] - d >= 0.0f);
     if (all_in) return n_in;
     const int dst = 1 - src;
     int n_out = 0;
-    float p0x = lds.x[src][n_in - 1][tid], p0y = lds.y[src][n_in - 1][tid];
-    float d0 = nx * p0x + ny * p0y - d;
+    real p0x = lds.x[src][n_in - 1][tid], p0y = lds.y[src][n_in - 1][tid];
+    real d0 = nx * p0x + ny * p0y - d;
     bool in0 = d0 >= 0.0f;
     for (int i = 0; i < n_in; i++) {
-        const float p1x = lds.x[src][i][tid], p1y = lds.y[src][i][tid];
-        const float d1 = nx * p1x + ny * p1y - d;
+        const real p1x = lds.x[src][i][tid], p1y = lds.y[src][i][tid];
+        const real d1 = nx * p1x + ny * p1y - d;
         const bool in1 = d1 >= 0.0f;
         // A convex polygon gains at most one vertex per pass (7 after four); the
         // capacity test only matters for slivers whose in/out pattern alternates
         // by rounding, where vertices beyond the eighth are dropped.
         if (in1 != in0 && n_out < kPolyCap) {
-            const float t = d0 / (d0 - d1);
+            const real t = d0 / (d0 - d1);
             lds.x[dst][n_out][tid] = p0x + t * (p1x - p0x);
             lds.y[dst][n_out][tid] = p0y + t * (p1y - p0y);
             n_out++;
@@ -98,7 +98,7 @@ __device__ __forceinline__ int owner_of_key(const uint32_t *__restrict__ tri_off
     return lo;
 }
 
-__global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__restrict__ vertices, int n_vertices,
+__global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                                const int32_t *__restrict__ indices, int n_triangles, int W,
                                                                int H, int tw, int th, int tiles_x, int tiles_y,
                                                                const uint32_t *__restrict__ tri_offsets, int64_t n_keys,
@@ -151,17 +151,17 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__r
     const int ty = r.y0 + (int)(local % ny);
 
     // render.cu:140-152 compute_plane
-    const float det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
-    const float id = (float)(1.0 / (double)det);
-    const float A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
-    const float B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
-    const float C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
+    const real det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+    const real id = (real)(1.0 / (double)det);
+    const real A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
+    const real B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
+    const real C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
 
     // render.cu:243-246 tile rectangle in NDC
-    const float xmin = (float)(tx * tw) / (float)W * 2.0f - 1.0f;
-    const float xmax = (float)((tx + 1) * tw) / (float)W * 2.0f - 1.0f;
-    const float ymin = (float)(ty * th) / (float)H * 2.0f - 1.0f;
-    const float ymax = (float)((ty + 1) * th) / (float)H * 2.0f - 1.0f;
+    const real xmin = (real)(tx * tw) / (real)W * 2.0f - 1.0f;
+    const real xmax = (real)((tx + 1) * tw) / (real)W * 2.0f - 1.0f;
+    const real ymin = (real)(ty * th) / (real)H * 2.0f - 1.0f;
+    const real ymax = (real)((ty + 1) * th) / (real)H * 2.0f - 1.0f;
 
     lds.x[0][0][tid] = p.ax; lds.y[0][0][tid] = p.ay;
     lds.x[0][1][tid] = p.bx; lds.y[0][1][tid] = p.by;
@@ -173,17 +173,22 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const float4 *__r
     if (n > 0) n = clip_pass(lds, cur, n, 0.0f, 1.0f, ymin);
     if (n > 0) n = clip_pass(lds, cur, n, 0.0f, -1.0f, -ymax);
 
-    float key = kFarKey;  // render.cu:259
+    real key = kFarKey;  // render.cu:259
     if (n > 0) {
-        float md = FLT_MAX;
+        real md = std::numeric_limits<real>::max();
         for (int i = 0; i < n; i++) {
-            const float pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
+            const real pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
             md = (pd < md) ? pd : md;
         }
         key = md;
     }
     const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
+#ifdef TG_DOUBLE_PRECISION
+    keys[k] = orderable_bits(key);  // all 64 bits are depth; the tile ids follow the depth keys
+    keys[n_keys + k] = tile;
+#else
     keys[k] = ((uint64_t)tile << 32) | orderable_bits(key);
+#endif
     payload[k] = (uint32_t)t;
 }
 
@@ -197,15 +202,15 @@ __global__ __launch_bounds__(kBinThreads) void tile_ranges_kernel(const uint64_t
 }
 
 // render.cu:310-337 cartesian_to_bary_kernel.
-__global__ __launch_bounds__(kBinThreads) void bary_kernel(const float4 *__restrict__ vertices, int n_vertices,
+__global__ __launch_bounds__(kBinThreads) void bary_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                            const int32_t *__restrict__ indices, int n_triangles,
-                                                           float *__restrict__ out) {
+                                                           real *__restrict__ out) {
     const int t = blockIdx.x * kBinThreads + threadIdx.x;
     if (t >= n_triangles) return;
     const TriXYZ p = load_triangle(vertices, n_vertices, indices, t);
-    float denom = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
-    if (fabsf(denom) < kEffZero) denom = 1.0f;
-    float *m = out + 9 * (int64_t)t;
+    real denom = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+    if (abs_real(denom) < kEffZero) denom = 1.0f;
+    real *m = out + 9 * (int64_t)t;
     m[0] = (p.by - p.cy) / denom;
     m[1] = (p.cx - p.bx) / denom;
     m[2] = (p.bx * p.cy - p.cx * p.by) / denom;
@@ -234,18 +239,18 @@ static int check_geometry(const char *fn, const void *vertices, int n_vertices, 
 
 using namespace tg;
 
-extern "C" int tg_bin_count(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+extern "C" int tg_bin_count(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
                             int tile_h, uint32_t *tri_counts, void *stream) {
     if (int e = check_geometry("tg_bin_count", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
     if (n_triangles == 0) return 0;
     if (!tri_counts) { set_error("tg_bin_count: tri_counts is null"); return TG_E_ARG; }
     TG_LAUNCH(bin_count_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
-                       (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
+                       (const real4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
                        ceil_div(width, tile_w), ceil_div(height, tile_h), tri_counts);
     return check_launch("bin_count_kernel");
 }
 
-extern "C" int tg_bin_emit(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
+extern "C" int tg_bin_emit(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width, int height, int tile_w,
                            int tile_h, const uint32_t *tri_offsets, int64_t n_keys, const uint32_t *owner_heads,
                            uint32_t owner_capacity, uint64_t *keys, uint32_t *payload, void *stream) {
     if (int e = check_geometry("tg_bin_emit", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
@@ -253,7 +258,7 @@ extern "C" int tg_bin_emit(const float *vertices, int32_t n_vertices, const int3
     if (n_keys == 0) return 0;
     if (n_triangles == 0 || !tri_offsets || !keys || !payload) { set_error("tg_bin_emit: null pointer"); return TG_E_ARG; }
     TG_LAUNCH(bin_emit_kernel, dim3((unsigned)ceil_div64(n_keys, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
-                       (const float4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
+                       (const real4 *)vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h,
                        ceil_div(width, tile_w), ceil_div(height, tile_h), tri_offsets, n_keys, owner_heads, owner_capacity, keys,
                        payload);
     return check_launch("bin_emit_kernel");
@@ -269,12 +274,12 @@ extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n
     return check_launch("tile_ranges_kernel");
 }
 
-extern "C" int tg_bary(const float *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, float *out,
+extern "C" int tg_bary(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, real *out,
                        void *stream) {
     if (int e = check_geometry("tg_bary", vertices, n_vertices, indices, n_triangles, 1, 1, 1, 1)) return e;
     if (n_triangles == 0) return 0;
     if (!out) { set_error("tg_bary: out is null"); return TG_E_ARG; }
     TG_LAUNCH(bary_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
-                       (const float4 *)vertices, n_vertices, indices, n_triangles, out);
+                       (const real4 *)vertices, n_vertices, indices, n_triangles, out);
     return check_launch("bary_kernel");
 }

@@ -4,20 +4,37 @@
 // (tile bounds, depth key, inside test, per-pixel depth, transmittance) is
 // evaluated exactly as the reference source writes it, one IEEE-754 operation
 // per source operator, no fused multiply-add.  The library must therefore be
-// compiled with -ffp-contract=off; float division is hipcc's correctly rounded
+// compiled with -ffp-contract=off; floating-point division is hipcc's correctly rounded
 // default.  Reference lines are relative to src/trigrad/ of the reference tree.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <cfloat>
+#include <limits>
 
 #include "../../include/trigrad_hip.h"
 
 namespace tg {
 
-constexpr float kEffZero = FLT_MIN;       // util.h:24
-constexpr float kMaxOpacity = 0.9999f;    // util.h:22
-constexpr float kFarKey = 1e30f;          // render.cu:259
+// The scalar type of the build (util.h:5-20): float, or double when the library
+// is compiled with -DTG_DOUBLE_PRECISION (the reference's DOUBLE_PRECISION).
+#ifdef TG_DOUBLE_PRECISION
+using real = double;
+using real4 = double4;
+#else
+using real = float;
+using real4 = float4;
+#endif
+static_assert(sizeof(real) == sizeof(tg_real), "the header's tg_real is the kernels' scalar type");
+__host__ __device__ __forceinline__ real4 make_real4(real x, real y, real z, real w) {
+    real4 v;
+    v.x = x; v.y = y; v.z = z; v.w = w;
+    return v;
+}
+
+constexpr real kEffZero = std::numeric_limits<real>::min();  // util.h:24
+constexpr real kMaxOpacity = (real)0.9999;                    // util.h:22
+constexpr real kFarKey = (real)1e30;                          // render.cu:259
 constexpr int kWave = 64;
 
 // ---- host side ---------------------------------------------------------------
@@ -46,37 +63,38 @@ inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // ---- device arithmetic ---------------------------------------------------------
 struct Rect { int x0, y0, x1, y1; };  // y0 == -1: the triangle touches no tile
 
-__device__ __forceinline__ float min3(float a, float b, float c) {
-    float m = a;
+__device__ __forceinline__ real min3(real a, real b, real c) {
+    real m = a;
     m = (b < m) ? b : m;
     m = (c < m) ? c : m;
     return m;
 }
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    float m = a;
+__device__ __forceinline__ real max3(real a, real b, real c) {
+    real m = a;
     m = (m < b) ? b : m;
     m = (m < c) ? c : m;
     return m;
 }
-__device__ __forceinline__ float clampf(float v, float lo, float hi) { return (v < lo) ? lo : ((hi < v) ? hi : v); }
+__host__ __device__ __forceinline__ real abs_real(real v) { return v < (real)0 ? -v : v; }
+__device__ __forceinline__ real clampf(real v, real lo, real hi) { return (v < lo) ? lo : ((hi < v) ? hi : v); }
 
 // Tile coordinate of an NDC coordinate (render.cu:72-75).  The 0.5 literal of
 // the source makes the product and quotient double precision.
-__device__ __forceinline__ int tile_coord(float m, int extent, int tile, int ntiles) {
-    float m1 = m + 1.0f;
+__device__ __forceinline__ int tile_coord(real m, int extent, int tile, int ntiles) {
+    real m1 = m + 1.0f;
     const double scaled = ((double)m1 * 0.5) * (double)extent;
     // dividing by a power of two is an exact scaling, so the reciprocal gives the same double
     const double t = ((tile & (tile - 1)) == 0) ? scaled * (1.0 / (double)tile) : scaled / (double)tile;
-    return (int)clampf((float)t, 0.0f, (float)(ntiles - 1));
+    return (int)clampf((real)t, 0.0f, (real)(ntiles - 1));
 }
 
 // render.cu:51-76 touched_tiles.
-__device__ __forceinline__ Rect tile_rect(float ax, float ay, float bx, float by, float cx, float cy, int W, int H, int tw,
+__device__ __forceinline__ Rect tile_rect(real ax, real ay, real bx, real by, real cx, real cy, int W, int H, int tw,
                                           int th, int tiles_x, int tiles_y) {
-    float ux = bx - ax, uy = by - ay, vx = cx - ax, vy = cy - ay;
-    float area2 = ux * vy - uy * vx;
+    real ux = bx - ax, uy = by - ay, vx = cx - ax, vy = cy - ay;
+    real area2 = ux * vy - uy * vx;
     Rect r;
-    if (fabsf(area2) < kEffZero || isnan(area2) || isinf(area2)) {
+    if (abs_real(area2) < kEffZero || isnan(area2) || isinf(area2)) {
         r.x0 = 0; r.y0 = -1; r.x1 = 0; r.y1 = -1;
         return r;
     }
@@ -90,35 +108,47 @@ __device__ __forceinline__ uint32_t rect_count(const Rect &r) {
     return (r.y0 == -1) ? 0u : (uint32_t)(r.x1 - r.x0 + 1) * (uint32_t)(r.y1 - r.y0 + 1);
 }
 
-// Order-preserving map float -> uint32 (ascending floats give ascending integers).
+// Order-preserving map of a floating-point value to an unsigned integer of the
+// same width (ascending values give ascending integers).
 __device__ __forceinline__ uint32_t orderable_bits(float f) {
     uint32_t b = __float_as_uint(f);
     return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
 }
+__device__ __forceinline__ uint64_t orderable_bits(double f) {
+    uint64_t b = (uint64_t)__double_as_longlong(f);
+    return b ^ ((b >> 63) ? ~0ull : (1ull << 63));
+}
+
+// An int carried in a slot of the scalar type, bit for bit.
+__device__ __forceinline__ float int_in_real(int v, float) { return __int_as_float(v); }
+__device__ __forceinline__ double int_in_real(int v, double) { return __longlong_as_double((long long)v); }
+__device__ __forceinline__ real int_in_real(int v) { return int_in_real(v, real()); }
+__device__ __forceinline__ int int_of_real(float v) { return __float_as_int(v); }
+__device__ __forceinline__ int int_of_real(double v) { return (int)__double_as_longlong(v); }
 
 // render.cu:78-88: bary = M * (x, y, 1).
-__device__ __forceinline__ void bary_apply(const float m[9], float px, float py, float &b0, float &b1, float &b2) {
+__device__ __forceinline__ void bary_apply(const real m[9], real px, real py, real &b0, real &b1, real &b2) {
     b0 = m[0] * px + m[1] * py + m[2];
     b1 = m[3] * px + m[4] * py + m[5];
     b2 = m[6] * px + m[7] * py + m[8];
 }
 // Strictly inside: all three at least FLT_MIN (render.cu:401, 438, 482).
-__device__ __forceinline__ bool bary_inside(float b0, float b1, float b2) {
+__device__ __forceinline__ bool bary_inside(real b0, real b1, real b2) {
     return !(b0 < kEffZero || b1 < kEffZero || b2 < kEffZero);
 }
 // util.h:245-250 interpolate3 with per-vertex weights.
-__device__ __forceinline__ float interp_w(float b0, float b1, float b2, float a, float b, float c, float w0, float w1, float w2) {
-    float denom = b0 * w0 + b1 * w1 + b2 * w2;
+__device__ __forceinline__ real interp_w(real b0, real b1, real b2, real a, real b, real c, real w0, real w1, real w2) {
+    real denom = b0 * w0 + b1 * w1 + b2 * w2;
     return (b0 * a * w0 + b1 * b * w1 + b2 * c * w2) / denom;
 }
 // Same with unit weights (multiplication by 1.0f is exact, so it is omitted).
-__device__ __forceinline__ float interp_1(float b0, float b1, float b2, float a, float b, float c) {
-    float denom = b0 + b1 + b2;
+__device__ __forceinline__ real interp_1(real b0, real b1, real b2, real a, real b, real c) {
+    real denom = b0 + b1 + b2;
     return (b0 * a + b1 * b + b2 * c) / denom;
 }
 // Pixel centre in NDC: double expression rounded once (render.cu:561-562).
-__device__ __forceinline__ float pixel_ndc(int i, int extent) {
-    return (float)(((double)(float)i + 0.5) / (double)(float)extent * 2.0 - 1.0);
+__device__ __forceinline__ real pixel_ndc(int i, int extent) {
+    return (real)(((double)(real)i + 0.5) / (double)(real)extent * 2.0 - 1.0);
 }
 
 // ---- wave64 DPP scan -----------------------------------------------------------

@@ -7,17 +7,20 @@
 // and mirror the arithmetic the backward kernels use on the device.
 #include <cfloat>
 #include <cmath>
+#include <limits>
 
 #include "../../include/trigrad_hip.h"
 
 namespace {
 
-constexpr float kTiny = FLT_MIN;  // util.h:24
+using real = tg_real;  // the scalar type of the build
 
-inline float cross2(float ax, float ay, float bx, float by) { return ax * by - ay * bx; }  // util.h:384-388
+constexpr real kTiny = std::numeric_limits<real>::min();  // util.h:24
 
-inline void bary_of(const float *v0, const float *v1, const float *v2, const float *p, float out[3]) {
-    const float T = cross2(v1[0] - v0[0], v1[1] - v0[1], v2[0] - v0[0], v2[1] - v0[1]);
+inline real cross2(real ax, real ay, real bx, real by) { return ax * by - ay * bx; }  // util.h:384-388
+
+inline void bary_of(const real *v0, const real *v1, const real *v2, const real *p, real out[3]) {
+    const real T = cross2(v1[0] - v0[0], v1[1] - v0[1], v2[0] - v0[0], v2[1] - v0[1]);
     out[0] = cross2(v1[0] - p[0], v1[1] - p[1], v2[0] - p[0], v2[1] - p[1]) / T;
     out[1] = cross2(v2[0] - p[0], v2[1] - p[1], v0[0] - p[0], v0[1] - p[1]) / T;
     out[2] = cross2(v0[0] - p[0], v0[1] - p[1], v1[0] - p[0], v1[1] - p[1]) / T;
@@ -26,23 +29,23 @@ inline void bary_of(const float *v0, const float *v1, const float *v2, const flo
 }  // namespace
 
 // util.h:395-403 barycentric(v0, v1, v2, p) -> 3 coordinates.
-extern "C" void tg_barycentric(const float *v0, const float *v1, const float *v2, const float *p, float *out) {
+extern "C" void tg_barycentric(const real *v0, const real *v1, const real *v2, const real *p, real *out) {
     bary_of(v0, v1, v2, p, out);
 }
 
 // util.h:405-455 barycentric_backward: grads (4 x 2, rows v0, v1, v2, p) of sum(g * bary).
-extern "C" void tg_barycentric_backward(const float *g, const float *a, const float *b, const float *c, const float *p,
-                                        float *grads) {
-    float l[3];
+extern "C" void tg_barycentric_backward(const real *g, const real *a, const real *b, const real *c, const real *p,
+                                        real *grads) {
+    real l[3];
     bary_of(a, b, c, p, l);
-    const float ax = a[0], ay = a[1], bx = b[0], by = b[1], cx = c[0], cy = c[1], px = p[0], py = p[1];
-    const float d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
+    const real ax = a[0], ay = a[1], bx = b[0], by = b[1], cx = c[0], cy = c[1], px = p[0], py = p[1];
+    const real d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
     if (std::fabs(d) < kTiny) {
         for (int i = 0; i < 8; i++) grads[i] = 0.0f;
         return;
     }
     // J[row][axis][k] = d bary_k / d row.axis
-    const float J[4][2][3] = {
+    const real J[4][2][3] = {
         {{l[0] * (-by + cy) / d, (-cy - l[1] * (by - cy) + py) / d, (by - l[2] * (by - cy) - py) / d},
          {l[0] * (bx - cx) / d, (cx + l[1] * (bx - cx) - px) / d, (-bx + l[2] * (bx - cx) + px) / d}},
         {{(cy + l[0] * (ay - cy) - py) / d, l[1] * (ay - cy) / d, (-ay + l[2] * (ay - cy) + py) / d},
@@ -56,22 +59,22 @@ extern "C" void tg_barycentric_backward(const float *g, const float *a, const fl
 }
 
 // util.h:245-250 scalar interpolate3 with weights.
-extern "C" float tg_interpolate3_scalar(const float *bary, float a, float b, float c, const float *w) {
-    const float denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
+extern "C" real tg_interpolate3_scalar(const real *bary, real a, real b, real c, const real *w) {
+    const real denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
     return (bary[0] * a * w[0] + bary[1] * b * w[1] + bary[2] * c * w[2]) / denom;
 }
 
 // util.h:299-317.  Outputs: grad_bary[3], grad_values[3] (a, b, c), grad_w[3].
-extern "C" void tg_interpolate3_scalar_backward(float g, const float *bary, float a, float b, float c, const float *w,
-                                                float *grad_bary, float *grad_values, float *grad_w) {
-    const float v[3] = {a, b, c};
-    const float nom = (bary[0] * w[0] * v[0] + bary[1] * w[1] * v[1]) + bary[2] * w[2] * v[2];
-    const float denom = (bary[0] * w[0] + bary[1] * w[1]) + bary[2] * w[2];
+extern "C" void tg_interpolate3_scalar_backward(real g, const real *bary, real a, real b, real c, const real *w,
+                                                real *grad_bary, real *grad_values, real *grad_w) {
+    const real v[3] = {a, b, c};
+    const real nom = (bary[0] * w[0] * v[0] + bary[1] * w[1] * v[1]) + bary[2] * w[2] * v[2];
+    const real denom = (bary[0] * w[0] + bary[1] * w[1]) + bary[2] * w[2];
     if (denom * denom < kTiny) {
         for (int k = 0; k < 3; k++) grad_bary[k] = grad_values[k] = grad_w[k] = 0.0f;
         return;
     }
-    const float inv2 = 1.0f / (denom * denom);
+    const real inv2 = 1.0f / (denom * denom);
     for (int k = 0; k < 3; k++) {
         grad_bary[k] = g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
         grad_values[k] = g * bary[k] * w[k] / denom;
@@ -80,27 +83,27 @@ extern "C" void tg_interpolate3_scalar_backward(float g, const float *bary, floa
 }
 
 // util.h:232-237 vector interpolate3 with weights (3 components).
-extern "C" void tg_interpolate3_vector(const float *bary, const float *a, const float *b, const float *c, const float *w,
-                                       float *out) {
-    const float denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
+extern "C" void tg_interpolate3_vector(const real *bary, const real *a, const real *b, const real *c, const real *w,
+                                       real *out) {
+    const real denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
     for (int k = 0; k < 3; k++) out[k] = (bary[0] * a[k] * w[0] + bary[1] * b[k] * w[1] + bary[2] * c[k] * w[2]) / denom;
 }
 
 // util.h:319-355.  Outputs: grad_bary[3], grad_a[3], grad_b[3], grad_c[3], grad_w[3].
-extern "C" void tg_interpolate3_vector_backward(const float *g, const float *bary, const float *a, const float *b,
-                                                const float *c, const float *w, float *grad_bary, float *grad_a,
-                                                float *grad_b, float *grad_c, float *grad_w) {
-    const float *v[3] = {a, b, c};
-    float nom[3];
+extern "C" void tg_interpolate3_vector_backward(const real *g, const real *bary, const real *a, const real *b,
+                                                const real *c, const real *w, real *grad_bary, real *grad_a,
+                                                real *grad_b, real *grad_c, real *grad_w) {
+    const real *v[3] = {a, b, c};
+    real nom[3];
     for (int k = 0; k < 3; k++) nom[k] = (bary[0] * w[0] * a[k] + bary[1] * w[1] * b[k]) + bary[2] * w[2] * c[k];
-    const float denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
+    const real denom = bary[0] * w[0] + bary[1] * w[1] + bary[2] * w[2];
     if (denom * denom < kTiny) {
         for (int k = 0; k < 3; k++) grad_bary[k] = grad_a[k] = grad_b[k] = grad_c[k] = grad_w[k] = 0.0f;
         return;
     }
-    const float inv2 = (float)(1.0 / (double)(denom * denom));
+    const real inv2 = (real)(1.0 / (double)(denom * denom));
     for (int i = 0; i < 3; i++) {
-        float dfb[3], dfw[3];
+        real dfb[3], dfw[3];
         for (int k = 0; k < 3; k++) {
             dfb[k] = w[i] * (v[i][k] * denom - nom[k]) * inv2;
             dfw[k] = (bary[i] * v[i][k] * denom - nom[k] * bary[i]) * inv2;
@@ -108,7 +111,7 @@ extern "C" void tg_interpolate3_vector_backward(const float *g, const float *bar
         grad_bary[i] = (g[0] * dfb[0] + g[1] * dfb[1]) + g[2] * dfb[2];
         grad_w[i] = (g[0] * dfw[0] + g[1] * dfw[1]) + g[2] * dfw[2];
     }
-    const float scale[3] = {bary[0] * w[0] / denom, bary[1] * w[1] / denom, bary[2] * w[2] / denom};
+    const real scale[3] = {bary[0] * w[0] / denom, bary[1] * w[1] / denom, bary[2] * w[2] / denom};
     for (int k = 0; k < 3; k++) {
         grad_a[k] = g[k] * scale[0];
         grad_b[k] = g[k] * scale[1];

@@ -17,18 +17,18 @@
 namespace tg {
 
 struct ForwardOut {
-    float4 *image;
-    float *depthmap;
-    float *weights;
+    real4 *image;
+    real *depthmap;
+    real *weights;
     int32_t *ends;
     int32_t *last;
-    float *last_depth;
+    real *last_depth;
     int32_t *fragments;  // (max_layers, H, W): list positions, relative to the tile's start, in blend order; may be null
 };
 
-__device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, float last_depth) {
+__device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, real last_depth) {
     // render.cu:609-618
-    float depth;
+    real depth;
     if (s.weight > kEffZero) {
         depth = s.depth / s.weight;
     } else {
@@ -40,7 +40,7 @@ __device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoor
     o.ends[p.index] = s.blended;
     if (o.last) o.last[p.index] = last;
     if (o.last_depth) o.last_depth[p.index] = last_depth;
-    o.image[p.index] = make_float4(s.c0, s.c1, s.c2, s.alpha);
+    o.image[p.index] = make_real4(s.c0, s.c1, s.c2, s.alpha);
 }
 
 __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(RasterArgs a, ForwardOut out) {
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
             if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
             if (e >= 0) {
                 const BlendRecord &r = s_rec[e];
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 blend_fragment(s, r, b0, b1, b2);
                 last = batch + e - start + 1;
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
 }
 
 // render.cu:338-373 insert_sorted_topk on an LDS candidate list of capacity `cap`.
-__device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, float d, int j) {
+__device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, real d, int j) {
     if (n == cap && d >= tk.d(cap - 1)) return;
     int i = (n < cap) ? n : cap - 1;
     while (i > 0 && d < tk.d(i - 1)) {
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
     const int n_threads = blockDim.x;
     DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
     TopK tk;
-    tk.depth = reinterpret_cast<float *>(s_dyn + sizeof(DepthRecord) * kBatch);
+    tk.depth = reinterpret_cast<real *>(s_dyn + sizeof(DepthRecord) * kBatch);
     tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
 
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
     publish_wave_rect(p, s_rects);
 
     PixelState s;
-    float last_depth = -__builtin_inff();  // render.cu:585-586
+    real last_depth = -__builtin_inff();  // render.cu:585-586
     int last_j = -1;
     bool active = p.valid;
     while (true) {
@@ -148,9 +148,9 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
                 if (e < 0) continue;
                 const DepthRecord &r = s_rec[e];
-                float b0, b1, b2;
+                real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                const float pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
+                const real pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
                 const int j = batch + e;
                 if (pd < last_depth) continue;
                 if (pd == last_depth && j <= last_j) continue;
@@ -163,15 +163,15 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         // apart: lanes reading different entries use different banks); entries
         // beyond it are gathered from memory.
         const int todo = (want && found > 0) ? min(found, a.max_layers - s.blended) : 0;
-        const float todo_depth = todo > 0 ? tk.d(todo - 1) : 0.0f;
+        const real todo_depth = todo > 0 ? tk.d(todo - 1) : 0.0f;
         __syncthreads();
-        float *rows = reinterpret_cast<float *>(s_dyn);
-        const int n_rows = min(end - start, (int)((sizeof(DepthRecord) * kBatch + sizeof(float) * kLayers * n_threads) /
-                                                   (sizeof(float) * kBlendWords)));
+        real *rows = reinterpret_cast<real *>(s_dyn);
+        const int n_rows = min(end - start, (int)((sizeof(DepthRecord) * kBatch + sizeof(real) * kLayers * n_threads) /
+                                                   (sizeof(real) * kBlendWords)));
         for (int e = tid; e < n_rows; e += blockDim.x) {
             BlendRecord r;
             gather_blend(a, start + e, r);
-            const float *w = reinterpret_cast<const float *>(&r);
+            const real *w = reinterpret_cast<const real *>(&r);
 #pragma unroll
             for (int k = 0; k < kBlendWords; k++) rows[e * kBlendWords + k] = w[k];
         }
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                     for (int u = 0; u < kGatherAhead; u++) {
                         const int rel = tk.j(min(i0 + u, todo - 1)) - start;
                         if (rel < n_rows) {
-                            float *w = reinterpret_cast<float *>(&r[u]);
+                            real *w = reinterpret_cast<real *>(&r[u]);
 #pragma unroll
                             for (int k = 0; k < kBlendWords; k++) w[k] = rows[rel * kBlendWords + k];
                         } else {
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
 #pragma unroll
                     for (int u = 0; u < kGatherAhead; u++) {
                         if (i0 + u >= todo) break;
-                        float b0, b1, b2;
+                        real b0, b1, b2;
                         bary_apply(r[u].m, p.px, p.py, b0, b1, b2);
                         if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
                         if (out.fragments) out.fragments[(int64_t)s.blended * ((int64_t)a.W * a.H) + p.index] = tk.j(i0 + u) - start;
@@ -241,7 +241,7 @@ int pixel_order_threads() {
 }
 
 size_t pixel_order_lds_bytes(int n_threads) {
-    return sizeof(DepthRecord) * kBatch + (size_t)kLayers * n_threads * (sizeof(float) + sizeof(int));
+    return sizeof(DepthRecord) * kBatch + (size_t)kLayers * n_threads * (sizeof(real) + sizeof(int));
 }
 
 // Dynamic LDS beyond 64 KB has to be enabled per kernel once.
@@ -276,11 +276,11 @@ int check_raster_args(const char *fn, int width, int height, int tile_w, int til
 
 using namespace tg;
 
-extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, const float *colors, const float *opacities,
-                                 const int32_t *sorted_ids, const int32_t *offsets, const float *bary, int width, int height,
-                                 int tile_w, int tile_h, float early_stopping_threshold, int per_pixel_sort, int max_layers,
-                                 float *image, float *depthmap, float *final_weights, int32_t *ends, int32_t *last,
-                                 float *last_depth, int32_t *fragments, void *stream) {
+extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, const real *colors, const real *opacities,
+                                 const int32_t *sorted_ids, const int32_t *offsets, const real *bary, int width, int height,
+                                 int tile_w, int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers,
+                                 real *image, real *depthmap, real *final_weights, int32_t *ends, int32_t *last,
+                                 real *last_depth, int32_t *fragments, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
         set_error("tg_render_forward: null pointer");
@@ -290,13 +290,13 @@ extern "C" int tg_render_forward(const float *vertices, const int32_t *indices, 
         set_error("tg_render_forward: vertices and image must be 16-byte aligned");
         return TG_E_ARG;
     }
-    RasterArgs a{(const float4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+    RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
     if (fragments && (!per_pixel_sort || max_layers > TG_MAX_SAVED_LAYERS)) {
         set_error("tg_render_forward: fragments are saved only with per_pixel_sort and max_layers <= %d", TG_MAX_SAVED_LAYERS);
         return TG_E_ARG;
     }
-    ForwardOut o{(float4 *)image, depthmap, final_weights, ends, last, last_depth, fragments};
+    ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments};
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads() : kTileThreads);
     const dim3 grid = tl.grid;
     const int n_threads = tl.threads;

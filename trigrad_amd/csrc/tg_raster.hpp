@@ -20,22 +20,22 @@ constexpr int kTileThreads = 256;     // workgroup size limit
 constexpr int kGatherAhead = 4;       // records a lane of a per-pixel-order kernel fetches together
 
 struct RasterArgs {
-    const float4 *vertices;
+    const real4 *vertices;
     const int32_t *indices;
-    const float *colors;
-    const float *opacities;
+    const real *colors;
+    const real *opacities;
     const int32_t *sorted_ids;
     const int32_t *offsets;
-    const float *bary;
+    const real *bary;
     int W, H, tw, th;
-    float thr;
+    real thr;
     int max_layers;
 };
 
 struct PixelCoord {
     int ix, iy, index;
     bool valid;
-    float px, py;
+    real px, py;
 };
 
 __device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
@@ -53,24 +53,24 @@ __device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
 
 // Everything process_forward (render.cu:417-453) reads for one list entry.
 struct alignas(16) BlendRecord {
-    float m[9];
-    float w[3];
-    float iw[3];   // 1/w per vertex (render.cu:444)
-    float op[3];
-    float col[9];  // vertex a rgb, vertex b rgb, vertex c rgb
-    float pad;
+    real m[9];
+    real w[3];
+    real iw[3];   // 1/w per vertex (render.cu:444)
+    real op[3];
+    real col[9];  // vertex a rgb, vertex b rgb, vertex c rgb
+    real pad;
 };
-static_assert(sizeof(BlendRecord) == 112, "BlendRecord layout");
-constexpr int kBlendWords = 27;  // floats of a BlendRecord without its padding; odd
+static_assert(sizeof(BlendRecord) == 28 * sizeof(real), "BlendRecord layout");
+constexpr int kBlendWords = 27;  // scalars of a BlendRecord without its padding; odd
 
 // What select_next_k_in_tile (render.cu:375-415) reads for one list entry.
 struct alignas(16) DepthRecord {
-    float m[9];
-    float z[3];
-    float w[3];
-    float pad;
+    real m[9];
+    real z[3];
+    real w[3];
+    real pad;
 };
-static_assert(sizeof(DepthRecord) == 64, "DepthRecord layout");
+static_assert(sizeof(DepthRecord) == 16 * sizeof(real), "DepthRecord layout");
 
 struct TriIds { int tri, ia, ib, ic; };
 
@@ -85,10 +85,10 @@ __device__ __forceinline__ TriIds load_ids(const RasterArgs &a, int j) {
 
 __device__ __forceinline__ void gather_blend(const RasterArgs &a, int j, BlendRecord &r) {
     const TriIds t = load_ids(a, j);
-    const float *m = a.bary + 9 * (int64_t)t.tri;
+    const real *m = a.bary + 9 * (int64_t)t.tri;
 #pragma unroll
     for (int k = 0; k < 9; k++) r.m[k] = m[k];
-    const float wa = a.vertices[t.ia].w, wb = a.vertices[t.ib].w, wc = a.vertices[t.ic].w;
+    const real wa = a.vertices[t.ia].w, wb = a.vertices[t.ib].w, wc = a.vertices[t.ic].w;
     r.w[0] = wa; r.w[1] = wb; r.w[2] = wc;
     r.iw[0] = 1.0f / wa; r.iw[1] = 1.0f / wb; r.iw[2] = 1.0f / wc;
     r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
@@ -102,29 +102,29 @@ __device__ __forceinline__ void gather_blend(const RasterArgs &a, int j, BlendRe
 
 __device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRecord &r) {
     const TriIds t = load_ids(a, j);
-    const float *m = a.bary + 9 * (int64_t)t.tri;
+    const real *m = a.bary + 9 * (int64_t)t.tri;
 #pragma unroll
     for (int k = 0; k < 9; k++) r.m[k] = m[k];
-    const float4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
+    const real4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
     r.z[0] = va.z; r.z[1] = vb.z; r.z[2] = vc.z;
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
 }
 
 // Front-to-back compositing state of one pixel (render.cu:564-574).
 struct PixelState {
-    float alpha = 1.0f, c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, depth = 0.0f, weight = 0.0f;
+    real alpha = 1.0f, c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, depth = 0.0f, weight = 0.0f;
     int blended = 0;
 };
 
 // The arithmetic of process_forward for a fragment known to be inside.
-__device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord &r, float b0, float b1, float b2) {
-    float o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], r.w[0], r.w[1], r.w[2]);
+__device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord &r, real b0, real b1, real b2) {
+    real o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], r.w[0], r.w[1], r.w[2]);
     o = clampf(o, 0.0f, kMaxOpacity);
-    const float k0 = interp_w(b0, b1, b2, r.col[0], r.col[3], r.col[6], r.w[0], r.w[1], r.w[2]);
-    const float k1 = interp_w(b0, b1, b2, r.col[1], r.col[4], r.col[7], r.w[0], r.w[1], r.w[2]);
-    const float k2 = interp_w(b0, b1, b2, r.col[2], r.col[5], r.col[8], r.w[0], r.w[1], r.w[2]);
-    const float z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
-    const float ao = s.alpha * o;
+    const real k0 = interp_w(b0, b1, b2, r.col[0], r.col[3], r.col[6], r.w[0], r.w[1], r.w[2]);
+    const real k1 = interp_w(b0, b1, b2, r.col[1], r.col[4], r.col[7], r.w[0], r.w[1], r.w[2]);
+    const real k2 = interp_w(b0, b1, b2, r.col[2], r.col[5], r.col[8], r.w[0], r.w[1], r.w[2]);
+    const real z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+    const real ao = s.alpha * o;
     s.depth = s.depth + ao * z;
     s.weight = s.weight + ao;
     s.c0 = s.c0 + ao * k0;
@@ -150,28 +150,30 @@ int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserv
 // evaluated with the same operations at the corner that maximises it, bounds
 // the value every pixel of the rectangle would compute.  If that bound is below
 // the inside threshold for one of the three coordinates, no lane can hit.
-struct WaveRect { float x_lo, x_hi, y_lo, y_hi; };
+struct WaveRect { real x_lo, x_hi, y_lo, y_hi; };
 
-__device__ __forceinline__ bool may_touch(const float m[9], const WaveRect &r) {
+__device__ __forceinline__ bool may_touch(const real m[9], const WaveRect &r) {
 #pragma unroll
     for (int k = 0; k < 3; k++) {
-        const float mx = m[3 * k], my = m[3 * k + 1];
-        const float x = (mx >= 0.0f) ? r.x_hi : r.x_lo;
-        const float y = (my >= 0.0f) ? r.y_hi : r.y_lo;
-        const float bound = mx * x + my * y + m[3 * k + 2];
+        const real mx = m[3 * k], my = m[3 * k + 1];
+        const real x = (mx >= 0.0f) ? r.x_hi : r.x_lo;
+        const real y = (my >= 0.0f) ? r.y_hi : r.y_lo;
+        const real bound = mx * x + my * y + m[3 * k + 2];
         if (bound < kEffZero) return false;  // a NaN bound never culls
     }
     return true;
 }
 
-__device__ __forceinline__ float wave_min(float v) {
+__device__ __forceinline__ real min_real(real a, real b) { return (b < a) ? b : a; }
+__device__ __forceinline__ real max_real(real a, real b) { return (a < b) ? b : a; }
+__device__ __forceinline__ real wave_min(real v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, kWave));
+    for (int off = 32; off > 0; off >>= 1) v = min_real(v, __shfl_xor(v, off, kWave));
     return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
+__device__ __forceinline__ real wave_max(real v) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    for (int off = 32; off > 0; off >>= 1) v = max_real(v, __shfl_xor(v, off, kWave));
     return v;
 }
 
@@ -180,7 +182,7 @@ constexpr int kMaxTileWaves = kTileThreads / kWave;
 // Every wave publishes the rectangle of its valid pixels (an empty rectangle,
 // lo > hi, if it has none); call with all threads, followed by __syncthreads().
 __device__ __forceinline__ void publish_wave_rect(const PixelCoord &p, WaveRect *s_rects) {
-    const float big = 3.0e38f;
+    const real big = 3.0e38f;
     WaveRect r;
     r.x_lo = wave_min(p.valid ? p.px : big);
     r.x_hi = wave_max(p.valid ? p.px : -big);
@@ -190,7 +192,7 @@ __device__ __forceinline__ void publish_wave_rect(const PixelCoord &p, WaveRect 
 }
 
 // Bit w of the result: wave w has to look at the entry.
-__device__ __forceinline__ uint32_t waves_touched(const float m[9], const WaveRect *s_rects, int n_waves) {
+__device__ __forceinline__ uint32_t waves_touched(const real m[9], const WaveRect *s_rects, int n_waves) {
     uint32_t bits = 0;
 #pragma unroll 1
     for (int w = 0; w < n_waves; w++) {
@@ -212,7 +214,7 @@ __device__ __forceinline__ uint64_t wave_candidates(const uint8_t *s_touch, int 
 // wave read the same record at the same time (LDS broadcast); only records that
 // can touch the wave's pixels are looked at.  Rec must have a member m[9].
 template <typename Rec>
-__device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *s_touch, int nb, int wave, float px, float py,
+__device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *s_touch, int nb, int wave, real px, real py,
                                                uint64_t m[kBatch / kWave]) {
 #pragma unroll
     for (int wd = 0; wd < kBatch / kWave; wd++) {
@@ -221,7 +223,7 @@ __device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *
         while (todo) {
             const int bit = __builtin_ctzll(todo);
             todo &= todo - 1;
-            float b0, b1, b2;
+            real b0, b1, b2;
             bary_apply(s_rec[wd * kWave + bit].m, px, py, b0, b1, b2);
             if (bary_inside(b0, b1, b2)) bits |= 1ull << bit;
         }
@@ -243,10 +245,10 @@ __device__ __forceinline__ int pop_lowest(uint64_t m[kBatch / kWave]) {
 // Per-pixel candidate lists of the per-pixel-sort mode live in LDS, slot-major:
 // entry `slot` of thread `t` is at [slot * n_threads + t] (conflict-free).
 struct TopK {
-    float *depth;
+    real *depth;
     int *pos;
     int n_threads;
-    __device__ __forceinline__ float &d(int slot) const { return depth[slot * n_threads + threadIdx.x]; }
+    __device__ __forceinline__ real &d(int slot) const { return depth[slot * n_threads + threadIdx.x]; }
     __device__ __forceinline__ int &j(int slot) const { return pos[slot * n_threads + threadIdx.x]; }
 };
 

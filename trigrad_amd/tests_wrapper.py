@@ -10,7 +10,7 @@ from torch.autograd import Function
 from . import _C, _lib
 from .util import create_check
 
-check_tensor = create_check("cpu", _C.precision)
+check_tensor = create_check("cpu", lambda: _C.precision)
 
 
 def _f(t):
@@ -19,8 +19,12 @@ def _f(t):
 
 
 def _out(n):
-    t = torch.empty((n,), dtype=torch.float32)
+    t = torch.empty((n,), dtype=_C.precision)
     return t, C.c_void_p(t.data_ptr())
+
+
+def _load():
+    return _lib.load(64 if _C.precision == torch.float64 else 32)
 
 
 class Barycentric(Function):
@@ -31,14 +35,14 @@ class Barycentric(Function):
         ctx.save_for_backward(p0, p1, q0, q1)
         keep = [_f(t) for t in (p0, p1, q0, q1)]
         out, po = _out(3)
-        _lib.load().tg_barycentric(*[p for _, p in keep], po)
+        _load().tg_barycentric(*[p for _, p in keep], po)
         return out
 
     @staticmethod
     def backward(ctx, grad_bary):
         keep = [_f(t) for t in (grad_bary, *ctx.saved_tensors)]
         grads, pg = _out(8)
-        _lib.load().tg_barycentric_backward(*[p for _, p in keep], pg)
+        _load().tg_barycentric_backward(*[p for _, p in keep], pg)
         g = grads.view(4, 2)
         return g[0].clone(), g[1].clone(), g[2].clone(), g[3].clone()
 
@@ -57,8 +61,8 @@ class Interpolate3Scalar(Function):
         check_tensor(w, "w", 3)
         ctx.save_for_backward(bary, a, b, c, w)
         kb, kw = _f(bary), _f(w)
-        val = _lib.load().tg_interpolate3_scalar(kb[1], float(a), float(b), float(c), kw[1])
-        return torch.tensor([val], dtype=torch.float32)
+        val = _load().tg_interpolate3_scalar(kb[1], float(a), float(b), float(c), kw[1])
+        return torch.tensor([val], dtype=_C.precision)
 
     @staticmethod
     def backward(ctx, grad_out):
@@ -67,7 +71,7 @@ class Interpolate3Scalar(Function):
         gb, pgb = _out(3)
         gv, pgv = _out(3)
         gw, pgw = _out(3)
-        _lib.load().tg_interpolate3_scalar_backward(float(grad_out), kb[1], float(a), float(b), float(c), kw[1], pgb, pgv, pgw)
+        _load().tg_interpolate3_scalar_backward(float(grad_out), kb[1], float(a), float(b), float(c), kw[1], pgb, pgv, pgw)
         return gb, gv[0:1].clone(), gv[1:2].clone(), gv[2:3].clone(), gw
 
 
@@ -83,14 +87,14 @@ class Interpolate3Vector(Function):
         ctx.save_for_backward(bary, a, b, c, w)
         keep = [_f(t) for t in (bary, a, b, c, w)]
         out, po = _out(3)
-        _lib.load().tg_interpolate3_vector(*[p for _, p in keep], po)
+        _load().tg_interpolate3_vector(*[p for _, p in keep], po)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         keep = [_f(t) for t in (grad_out, *ctx.saved_tensors)]
         outs = [_out(3) for _ in range(5)]
-        _lib.load().tg_interpolate3_vector_backward(*[p for _, p in keep], *[p for _, p in outs])
+        _load().tg_interpolate3_vector_backward(*[p for _, p in keep], *[p for _, p in outs])
         return tuple(t for t, _ in outs)  # grad_bary, grad_a, grad_b, grad_c, grad_w
 
 

@@ -8,8 +8,8 @@ from torch.autograd import Function
 from . import _C
 from .util import create_check
 
-check_tensor = create_check("cuda", _C.precision)
-precision = _C.precision
+check_tensor = create_check("cuda", lambda: _C.precision)
+precision = _C.precision  # the scalar type at import (TRIGRAD_PRECISION); _C.set_precision changes what the checks expect
 
 
 class Renderer(Function):
