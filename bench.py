@@ -5,7 +5,7 @@
 
 A step is one forward + backward pass of `trigrad_amd.render` (L2 loss against a
 seeded random target) over one synthetic frame that is already resident in HBM.
-The default workload is configuration 2 of BASELINE.json (1,000,000 triangles,
+The default workload is the headline configuration (1,000,000 triangles,
 1920x1080, float32, 16x16 tiles).  One JSON line is printed:
 
   value            forward+backward frames/s (the headline metric)
