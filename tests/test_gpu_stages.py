@@ -108,7 +108,8 @@ def test_binning_sort_ranges_bit_exact(name, cuda, oracle):
     np.testing.assert_array_equal(got_bary.view(np.uint32), want_bary.view(np.uint32))
 
 
-@pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 2047, 2048, 2049, 100_003, (1 << 20) + 7])
+# the largest size has more tiles than workgroups fit the device at once (ticketed tile numbers)
+@pytest.mark.parametrize("n", [1, 5, 63, 64, 65, 2047, 2048, 2049, 100_003, (1 << 20) + 7, 6_000_011])
 def test_scan_matches_cumsum(n, cuda):
     import torch
     from trigrad_amd import _C
@@ -135,6 +136,7 @@ def test_scan_empty(cuda):
 @pytest.mark.parametrize("n,end_bit,distinct", [
     (1, 64, None), (2, 64, None), (100, 64, None), (4095, 64, None), (4096, 64, None), (4097, 64, None),
     (100_000, 64, None), (100_000, 45, None), (50_000, 64, 7), (300_000, 40, 1000), ((1 << 20) + 13, 45, None),
+    (5_000_017, 45, None), (5_000_017, 24, 50_000),  # more tiles than fit the device at once: ticketed tile numbers
 ])
 def test_sort_pairs_stable(n, end_bit, distinct, cuda, oracle):
     """Random keys, optionally drawn from few distinct values so that stability

@@ -56,6 +56,23 @@ ProfileScope::~ProfileScope() {
     if (slot < (int)g_profile_records.size()) (void)hipEventRecord(g_profile_records[slot].stop, stream);
 }
 
+int resident_workgroups(const void *kernel, int threads, int *cache) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    if (cache[dev] == 0) {
+        int per_cu = 0;
+        hipDeviceProp_t prop;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess ||
+            hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            cache[dev] = -1;
+        } else {
+            cache[dev] = per_cu * prop.multiProcessorCount > 0 ? per_cu * prop.multiProcessorCount : -1;
+        }
+    }
+    return cache[dev] > 0 ? cache[dev] : 0;
+}
+
 }  // namespace tg
 
 extern "C" int tg_version(void) { return TG_ABI_VERSION; }

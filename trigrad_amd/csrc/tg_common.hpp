@@ -57,6 +57,13 @@ struct ProfileScope {
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__); \
     } while (0)
 
+// Workgroups of `kernel` that can be resident on the current device at once
+// (0 if unknown).  A grid that is no larger needs no ticket to number its
+// workgroups for a look-back chain: every workgroup is started without waiting
+// for another to finish, so waiting on lower-numbered ones cannot deadlock.
+int resident_workgroups(const void *kernel, int threads, int *cache /* [kMaxDevices] */);
+constexpr int kMaxDevices = 64;
+
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

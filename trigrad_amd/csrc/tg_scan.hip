@@ -10,7 +10,8 @@
 // ready, 2 inclusive prefix ready; bits 31..0 = the value.  Value and flag
 // share one word, so relaxed agent-scope atomic loads/stores are sufficient.
 // Tiles are numbered by an atomic ticket taken at workgroup start, so every
-// tile a workgroup waits for is already running.  The wait is bounded: on
+// tile a workgroup waits for is already running; a grid that fits the device
+// at once uses the workgroup ids instead.  The wait is bounded: on
 // expiry the kernel records TG_STATUS_LOOKBACK_TIMEOUT and carries on (with a
 // wrong result) so that every wave still exits.
 #include "tg_common.hpp"
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint3
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
     __syncthreads();
     const int tile = (int)s_tile;
 
@@ -174,6 +175,8 @@ extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t 
     TG_LAUNCH(scan_init_kernel, dim3(init_blocks), dim3(256), 0, s, ticket, states, n_tiles, total, status);
     if (int e = check_launch("scan_init_kernel")) return e;
     if (n_tiles == 0) return 0;
+    static int resident_cache[kMaxDevices] = {0};
+    if (n_tiles <= resident_workgroups((const void *)scan_lookback_kernel, kScanThreads, resident_cache)) ticket = nullptr;
     TG_LAUNCH(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
                        n_tiles, status, head_stride, head_capacity, heads);
     return check_launch("scan_lookback_kernel");

@@ -25,7 +25,10 @@
 //                   digit run is written contiguously.
 //
 // Tiles are numbered by an atomic ticket so that a workgroup only ever waits for
-// workgroups that already run; waits are bounded (TG_STATUS_LOOKBACK_TIMEOUT).
+// workgroups that already run -- or, when the whole grid fits the device at once
+// (then no workgroup has to finish for another to start), by the workgroup ids,
+// which saves the serialised same-address atomics.  Waits are bounded
+// (TG_STATUS_LOOKBACK_TIMEOUT).
 #include "tg_common.hpp"
 
 namespace tg {
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
     for (int w = 0; w < kSortWaves; w++) s_wave_count[w][tid] = 0;
     __syncthreads();
     const int tile = (int)s_tile;
@@ -352,9 +355,14 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
 
     uint64_t *kin = keys, *kout = keys_alt;
     uint32_t *vin = values, *vout = values_alt;
+    // 534 same-address ticket atomics cost 6 us per pass; a grid that fits the device whole takes its
+    // tile numbers from the workgroup ids instead
+    static int resident_cache[kMaxDevices] = {0};
+    const bool whole_grid_resident = L.n_tiles <= resident_workgroups((const void *)sort_sweep_kernel, kSortThreads, resident_cache);
     for (int p = 0; p < L.passes; p++) {
         TG_LAUNCH(sort_sweep_kernel, dim3(L.n_tiles), dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, p * kRadixBits,
-                           bases + p * kRadix, lookback + (size_t)p * L.n_tiles * kRadix, tickets + p, status);
+                           bases + p * kRadix, lookback + (size_t)p * L.n_tiles * kRadix,
+                           whole_grid_resident ? (uint32_t *)nullptr : tickets + p, status);
         if (int e = check_launch("sort_sweep_kernel")) return e;
         uint64_t *tk = kin; kin = kout; kout = tk;
         uint32_t *tv = vin; vin = vout; vout = tv;
