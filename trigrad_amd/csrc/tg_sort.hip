@@ -42,7 +42,7 @@ constexpr int kSortItems = 16;
 constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
 constexpr int kHistBlocksMax = 256;
 constexpr int kBasesThreads = 1024;
-constexpr int kLookWindow = 16;
+constexpr int kLookWindow = 4;  // predecessors read per round trip; wider windows only add L2 traffic (measured 1..64)
 constexpr uint32_t kSortSpinLimit = 1u << 20;
 constexpr uint32_t kLbAggregate = 1u << 30;
 constexpr uint32_t kLbInclusive = 2u << 30;
