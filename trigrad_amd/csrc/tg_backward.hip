@@ -760,7 +760,7 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
         TG_LAUNCH(backward_saved_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
         return check_launch("backward_saved_order_kernel");
     }
-    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads());
+    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads(kTileThreads));
     const size_t lds = backward_pixel_order_lds_bytes(tl.threads);
     static size_t lds_reserved = 0;
     if (int e = reserve_lds("tg_render_backward", (const void *)backward_pixel_order_kernel, lds, &lds_reserved)) return e;

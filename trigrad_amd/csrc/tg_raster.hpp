@@ -137,7 +137,7 @@ __device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord 
 // ---- host-side launch helpers (defined in tg_forward.hip) ---------------------------
 struct TileLaunch { dim3 grid; int threads; };
 TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads);
-int pixel_order_threads();
+int pixel_order_threads(int preferred);
 size_t pixel_order_lds_bytes(int n_threads);
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
 int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
