@@ -261,6 +261,38 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
     return st;
 }
 
+// Adds up, in slot order, the runs of equal tag among slots [c0, c1) of one row
+// of a term matrix and hands every non-zero run sum to flush(tag, sum).  Tags and
+// terms are read eight slots ahead, so the LDS latency is paid once per eight
+// slots instead of once per slot.
+template <typename TagAt, typename Flush>
+__device__ __forceinline__ void sum_runs(const real *row, int c0, int c1, TagAt tag_at, Flush flush) {
+    constexpr int kAhead = 8;
+    int cur = tag_at(c0);
+    real sum = 0.0f;
+    for (int c = c0; c < c1; c += kAhead) {
+        int t[kAhead];
+        real v[kAhead];
+#pragma unroll
+        for (int k = 0; k < kAhead; k++) {
+            const int i = min(c + k, c1 - 1);
+            t[k] = tag_at(i);
+            v[k] = row[i];
+        }
+#pragma unroll
+        for (int k = 0; k < kAhead; k++) {
+            if (c + k >= c1) break;
+            if (t[k] != cur) {
+                if (sum != 0.0f) flush(cur, sum);
+                sum = 0.0f;
+                cur = t[k];
+            }
+            sum += v[k];
+        }
+    }
+    if (sum != 0.0f) flush(cur, sum);
+}
+
 constexpr int kBackBatch = 128;   // list entries staged per batch
 constexpr int kWaveSlots = 256;   // hit slots per wave and round
 constexpr int kSeedWords = 6;     // d_do, gc[3], dd_dz, (entry | source lane << 8)
@@ -446,20 +478,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 const int group = lane / kTerms, q = lane - group * kTerms;
                 const int per = (n_here + 2) / 3;
                 const int c0 = group * per, c1 = min(c0 + per, n_here);
-                if (group < 3 && c0 < c1) {
-                    int cur = int_of_real(seeds[5][s0 + c0]) & 0xff;
-                    real acc = 0.0f;
-                    for (int c = c0; c < c1; c++) {
-                        const int t = int_of_real(seeds[5][s0 + c]) & 0xff;
-                        if (t != cur) {
-                            if (acc != 0.0f) unsafeAtomicAdd(term_address(g, s_rec[cur].id[q / 7], q % 7), acc);
-                            acc = 0.0f;
-                            cur = t;
-                        }
-                        acc += terms[q * kTermStride + c];
-                    }
-                    if (acc != 0.0f) unsafeAtomicAdd(term_address(g, s_rec[cur].id[q / 7], q % 7), acc);
-                }
+                if (group < 3 && c0 < c1)
+                    sum_runs(terms + q * kTermStride, c0, c1,
+                             [&](int c) { return int_of_real(seeds[5][s0 + c]) & 0xff; },
+                             [&](int entry, real sum) { unsafeAtomicAdd(term_address(g, s_rec[entry].id[q / 7], q % 7), sum); });
                 wave_lds_sync();
             }
         }
@@ -696,22 +718,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
             const int group = lane / kTerms, q = lane - group * kTerms;
             const int per = (n_slots + 2) / 3;
             const int c0 = group * per, c1 = min(c0 + per, n_slots);
-            if (group < 3 && c0 < c1) {
-                int cur = tags[c0];
-                real sum = 0.0f;
-                for (int c = c0; c < c1; c++) {
-                    const int t = tags[c];
-                    if (t != cur) {
-                        if (sum != 0.0f)
-                            unsafeAtomicAdd(term_address(g, int_of_real(s_rows[cur * kSavedStride + kBackReals + q / 7]), q % 7), sum);
-                        sum = 0.0f;
-                        cur = t;
-                    }
-                    sum += terms[q * kTermStride + c];
-                }
-                if (sum != 0.0f)
-                    unsafeAtomicAdd(term_address(g, int_of_real(s_rows[cur * kSavedStride + kBackReals + q / 7]), q % 7), sum);
-            }
+            if (group < 3 && c0 < c1)
+                sum_runs(terms + q * kTermStride, c0, c1, [&](int c) { return tags[c]; }, [&](int entry, real sum) {
+                    unsafeAtomicAdd(term_address(g, int_of_real(s_rows[entry * kSavedStride + kBackReals + q / 7]), q % 7), sum);
+                });
             wave_lds_sync();
         }
     }
