@@ -85,10 +85,11 @@ __device__ __forceinline__ void interp_backward_scalar(real g, const real b[3], 
         return;
     }
     const real inv2 = 1.0f / (denom * denom);
+    const real inv = 1.0f / denom;  // shared by the three value gradients (the reference divides three times)
 #pragma unroll
     for (int k = 0; k < 3; k++) {
         gb[k] = g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
-        gv[k] = g * b[k] * w[k] / denom;
+        gv[k] = g * b[k] * w[k] * inv;
         gw[k] = g * (b[k] * v[k] * denom - nom * b[k]) * inv2;
     }
 }
@@ -161,6 +162,7 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
         const real denom = b[0] * w[0] + b[1] * w[1] + b[2] * w[2];
         if (!(denom * denom < kEffZero)) {
             const real inv2 = 1.0f / (denom * denom);
+            const real inv = 1.0f / denom;
 #pragma unroll
             for (int v = 0; v < 3; v++) {
                 real dfb[3], dfw[3];
@@ -172,7 +174,7 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
                 }
                 gb_c[v] = (gc[0] * dfb[0] + gc[1] * dfb[1]) + gc[2] * dfb[2];
                 gw_c[v] = (gc[0] * dfw[0] + gc[1] * dfw[1]) + gc[2] * dfw[2];
-                scale[v] = b[v] * w[v] / denom;
+                scale[v] = b[v] * w[v] * inv;
             }
         }
     }
