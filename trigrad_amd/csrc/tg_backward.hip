@@ -118,18 +118,19 @@ __device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const Bac
     const real z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
 
     const real om = 1.0f - o;
+    const real inv_om = 1.0f / om;  // the reference divides six derivative terms by om; they share this reciprocal
     const real g[3] = {st.g0, st.g1, st.g2};
     real s[3] = {st.s0, st.s1, st.s2};
     real t3[3];
 #pragma unroll
-    for (int k = 0; k < 3; k++) t3[k] = (color[k] * st.alpha - s[k]) / om * g[k];
-    const real drgb_do = ((t3[0] + t3[1]) + t3[2]) + st.g3 * (-st.final_alpha / om);  // :491
-    st.alpha /= om;                                                                    // :492
+    for (int k = 0; k < 3; k++) t3[k] = (color[k] * st.alpha - s[k]) * inv_om * g[k];
+    const real drgb_do = ((t3[0] + t3[1]) + t3[2]) + st.g3 * (-st.final_alpha * inv_om);  // :491
+    st.alpha /= om;                                                                        // :492 (state: kept exact)
 #pragma unroll
     for (int k = 0; k < 3; k++) s[k] += color[k] * o * st.alpha;                       // :493
     st.s0 = s[0]; st.s1 = s[1]; st.s2 = s[2];
-    const real ddw_do = st.alpha - st.oa / om;                                        // :494
-    const real dud_do = st.alpha * z - st.zoa / om;                                   // :495
+    const real ddw_do = st.alpha - st.oa * inv_om;                                    // :494
+    const real dud_do = st.alpha * z - st.zoa * inv_om;                               // :495
     st.oa = st.oa + o * st.alpha;                                                      // :496
     st.zoa = st.zoa + z * o * st.alpha;                                                // :497
     real dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
