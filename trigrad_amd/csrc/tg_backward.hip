@@ -69,6 +69,7 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
 // Reverse-traversal state of one pixel (render.cu:647-653).
 struct BackState {
     real final_alpha, alpha, s0, s1, s2, oa, zoa, final_weight, final_depth;
+    real inv_final_weight;  // the reference divides two terms of every fragment by the pixel's final weight
     real g0, g1, g2, g3, gd;  // upstream gradient of this pixel
 };
 
@@ -110,11 +111,16 @@ struct FragSeed {
 
 __device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, real b0, real b1, real b2) {
     const real w[3] = {r.w[0], r.w[1], r.w[2]};
+    // The opacity is recomputed exactly as the forward pass computed it: 1 - o can be small, and the
+    // transmittance is reconstructed by dividing by it.  The three colour quotients over the same
+    // denominator (util.h:245-250) share its reciprocal.
     real o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
     o = clampf(o, 0.0f, kMaxOpacity);
+    const real inv_denom = 1.0f / (b0 * w[0] + b1 * w[1] + b2 * w[2]);
     real color[3];
 #pragma unroll
-    for (int k = 0; k < 3; k++) color[k] = interp_w(b0, b1, b2, r.col[k], r.col[3 + k], r.col[6 + k], w[0], w[1], w[2]);
+    for (int k = 0; k < 3; k++)
+        color[k] = (b0 * r.col[k] * w[0] + b1 * r.col[3 + k] * w[1] + b2 * r.col[6 + k] * w[2]) * inv_denom;
     const real z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
 
     const real om = 1.0f - o;
@@ -133,13 +139,13 @@ __device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const Bac
     const real dud_do = st.alpha * z - st.zoa * inv_om;                               // :495
     st.oa = st.oa + o * st.alpha;                                                      // :496
     st.zoa = st.zoa + z * o * st.alpha;                                                // :497
-    real dd_do = (dud_do - st.final_depth * ddw_do) / st.final_weight * st.gd;        // :499
+    real dd_do = (dud_do - st.final_depth * ddw_do) * st.inv_final_weight * st.gd;    // :499
     if (st.final_weight < kEffZero) dd_do = 0.0f;
     FragSeed f;
     f.d_do = drgb_do + dd_do;
     const real ao = st.alpha * o;
     f.gc[0] = ao * g[0]; f.gc[1] = ao * g[1]; f.gc[2] = ao * g[2];                     // :510
-    f.dd_dz = ao * st.gd / st.final_weight;                                            // :517
+    f.dd_dz = ao * st.gd * st.inv_final_weight;                                        // :517
     if (st.final_weight < kEffZero) f.dd_dz = 0.0f;
     return f;
 }
@@ -265,6 +271,7 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
     st.s0 = st.s1 = st.s2 = 0.0f;
     st.oa = st.zoa = 0.0f;
     st.final_weight = g.weights[p.index];
+    st.inv_final_weight = 1.0f / st.final_weight;
     st.final_depth = g.depthmap[p.index];
     return st;
 }
