@@ -4,17 +4,20 @@
 // of a fragment is reconstructed by dividing the running value by (1 - opacity),
 // as the reference does (render.cu:492).
 //
-// per_pixel_sort = 0: all pixels of a tile share the list order, so the tile's
-//   list is walked backwards in LDS-staged batches.  Each fragment yields 21
-//   gradient terms (3 vertices x {x, y, w, r, g, b, opacity}; the z gradient is
-//   identically zero, render.cu:531-533).  They are summed per list entry in
-//   LDS (wave-level DPP reduction when many lanes of a wave hit the same entry,
-//   LDS real atomics otherwise) and flushed with at most 21 global real
-//   atomics per (tile, entry) instead of 24 per (pixel, entry).
-// per_pixel_sort = 1: every pixel has its own order; the pixel re-selects its
-//   fragments from the far end (32 at a time, below the (depth, position) of the
-//   last blended fragment saved by the forward pass) and issues its atomics
-//   directly.
+// Each fragment yields 21 gradient terms (3 vertices x {x, y, w, r, g, b,
+// opacity}; the z gradient is identically zero, render.cu:531-533).  Terms of
+// the same list entry are added up inside a wave before they reach memory, so
+// the kernels issue one global floating-point atomic per (wave, run of equal
+// entries, term) instead of 24 per (pixel, entry).
+//
+// per_pixel_sort = 0 (backward_tile_order_kernel): all pixels of a tile share
+//   the list order, so the tile's list is walked backwards in LDS-staged
+//   batches of 128 entries.
+// per_pixel_sort = 1, max_layers <= 32 (backward_saved_order_kernel): every
+//   pixel walks the blend order the forward pass saved for it, backwards.
+// per_pixel_sort = 1, max_layers > 32 (backward_pixel_order_kernel): the pixel
+//   re-selects its fragments from the far end (32 at a time, below the (depth,
+//   position) of the last blended fragment saved by the forward pass).
 #include "tg_raster.hpp"
 
 namespace tg {
@@ -329,7 +332,7 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Tile-order backward.  LDS real atomics cost about three cycles per lane on
+// Tile-order backward.  LDS floating-point atomics cost about three cycles per lane on
 // gfx950 and direct global atomics collide on the shared vertices, so the
 // per-entry sums are formed with plain LDS stores and loads.  The records of
 // 128 list entries are staged per batch by the whole workgroup; after that
@@ -347,7 +350,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 //   4. order-free part, 64 slots at a time with every lane busy: lane = slot
 //      evaluates the 21 gradient terms of its hit and writes them to a term
 //      matrix; three groups of 21 lanes add up the runs of equal entry and issue
-//      one global real atomic per run and term.
+//      one global floating-point atomic per run and term.
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ BackRecord s_rec[kBackBatch];
     __shared__ uint64_t s_ballot[kMaxWaves][kBackBatch];
@@ -632,12 +635,12 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 // kSavedWindow list entries of the tile are staged once (rows an odd number of
 // words apart, so lanes reading different entries use different banks).  Every
 // wave walks its 64 pixels in lockstep, each lane from its own far end.  LDS
-// real atomics cost about three cycles per lane on gfx950 and many lanes of a
+// floating-point atomics cost about three cycles per lane on gfx950 and many lanes of a
 // wave hold the same entry in the same step, so the 21 gradient terms of a step
 // are grouped by entry first: lanes with equal entries get consecutive slots
 // (ballot matching, groups in order of their lowest lane), the terms go to a
 // slot-major matrix in LDS, three groups of 21 lanes add up the runs of equal
-// entry and issue one global real atomic per run and term.  Fragments of
+// entry and issue one global floating-point atomic per run and term.  Fragments of
 // entries beyond the staged window are gathered from and added to memory
 // directly.
 constexpr int kSavedWindow = 256;

@@ -1,11 +1,13 @@
 // tg_binning.hip -- tile binning (count, key emission), tile ranges and bary matrices.
 //
-// All four kernels are HBM-bound streaming kernels:
+// count, ranges and bary are HBM-bound streaming kernels; emit is bound by the
+// clipping arithmetic it does per key:
 //   count   reads 12 B indices + 3 x 16 B vertex gathers, writes 4 B per triangle
 //   emit    one thread per KEY (not per triangle), so a triangle that covers
 //           thousands of tiles is spread over thousands of lanes; reads the
-//           triangle again (L2 hits for neighbouring keys), writes 8 B key +
-//           4 B payload per key, coalesced
+//           triangle again (L2 hits for neighbouring keys), clips it to the
+//           tile (polygon in LDS), writes 8 B key + 4 B payload per key,
+//           coalesced
 //   ranges  reads 8 B per sorted key, writes 4 B per tile
 //   bary    reads 60 B, writes 36 B per triangle
 #include "tg_common.hpp"
