@@ -270,7 +270,18 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
         heads = owner_heads_for(indices.shape[0], dev)
         tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
-        host = total._base.cpu()
+        bary_transforms = None
+        if disable_timing:
+            # K travels to pinned host memory while the device already computes the bary matrices, which do
+            # not depend on it; the host waits for the copy only (with stage timings the reference's order is kept)
+            host = torch.empty((2,), dtype=torch.int32, pin_memory=True)
+            host.copy_(total._base, non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+            bary_transforms = cartesian_to_bary(vertices, indices)
+            arrived.synchronize()
+        else:
+            host = total._base.cpu()
         K, st = int(host[0]), int(host[1])
         if st != 0:
             raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
@@ -280,7 +291,8 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
         keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
 
         timer.start("bary_transforms")
-        bary_transforms = cartesian_to_bary(vertices, indices)
+        if bary_transforms is None:
+            bary_transforms = cartesian_to_bary(vertices, indices)
 
         timer.start("rasterization")
         _lib.check(lib.tg_render_forward(
