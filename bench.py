@@ -154,6 +154,16 @@ def main():
                                 "frac_of_hbm_peak": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS},
         "sort_in_frame": {"keys": K, "passes": passes, "ms": sort_ms, "Gkeys_per_s": K / (sort_ms / 1000.0) / 1e9},
     }
+    # the blend kernels against the HBM roofline, to show that it does not bound them: compulsory bytes are
+    # 148 B per list entry plus the per-pixel and per-vertex arrays (forward 28 B/pixel; backward 48 B/pixel + 64 B/vertex)
+    V, P = d["vertices"].shape[0], W * H
+    blend = {}
+    for name, nbytes in (("forward", 148.0 * K + 28.0 * P), ("backward", 148.0 * K + 48.0 * P + 64.0 * V)):
+        kms = sum(v for k, v in per_step.items() if k.startswith(name))
+        if kms > 0:
+            blend[name] = {"ms": kms, "compulsory_bytes": nbytes, "GBps": nbytes / (kms / 1000.0) / 1e9,
+                           "frac_of_hbm_peak": nbytes / (kms / 1000.0) / 1e9 / HBM_PEAK_GBS, "bound": "vector issue / LDS, not HBM"}
+    extra["blend_kernels_vs_hbm"] = blend
     if not args.no_extras:
         extra["forward_only_fps"] = 1000.0 / timed(lambda: step(args.mode, backward=False), args.steps, 1)
         other = "A" if args.mode == "B" else "B"
