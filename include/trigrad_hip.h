@@ -154,12 +154,17 @@ int tg_bary(const tg_real *vertices, int32_t n_vertices, const int32_t *indices,
  * in blend order (layer k of pixel p at fragments[k*H*W + p], k < ends[p]);
  * tg_render_backward then walks them backwards instead of selecting the
  * fragments again (the reference re-selects, render.cu:667-693).
+ * hit_masks (tg_hit_mask_words() uint64 words), or NULL: without per_pixel_sort
+ * the kernel also writes, for every pixel and every 64 consecutive entries of
+ * its tile's list that it looked at, which of them cover the pixel;
+ * tg_render_backward then reads them back instead of repeating the inside tests.
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
+size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int tile_w, int tile_h);
 int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_real *colors, const tg_real *opacities,
                       const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, int width, int height,
                       int tile_w, int tile_h, tg_real early_stopping_threshold, int per_pixel_sort, int max_layers,
                       tg_real *image, tg_real *depthmap, tg_real *final_weights, int32_t *ends, int32_t *last,
-                      tg_real *last_depth, int32_t *fragments, void *stream);
+                      tg_real *last_depth, int32_t *fragments, uint64_t *hit_masks, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
 
@@ -167,13 +172,14 @@ int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_
  * which the caller zero-initialises.  Replaces render_backward_kernel /
  * process_backward (render.cu:455-538, 621-695).  Fragments are visited in
  * exact reverse blend order.  grad_depthmap may be NULL (= all zero: the depth
- * map took no part in the loss).  fragments: what tg_render_forward saved, or
- * NULL (then last and, with per_pixel_sort, last_depth locate the far end). */
+ * map took no part in the loss).  fragments, hit_masks: what tg_render_forward
+ * saved, or NULL (then the fragments are selected, the inside tests made again). */
 int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, const tg_real *vertices,
                        const int32_t *indices, const tg_real *colors, const tg_real *opacities,
                        const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, const tg_real *image,
                        const tg_real *depthmap, const tg_real *final_weights, const int32_t *ends, const int32_t *last,
-                       const tg_real *last_depth, const int32_t *fragments, int width, int height, int tile_w, int tile_h,
+                       const tg_real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width, int height,
+                       int tile_w, int tile_h,
                        tg_real early_stopping_threshold, int per_pixel_sort, int max_layers, tg_real *grad_vertices,
                        tg_real *grad_colors, tg_real *grad_opacities, void *stream);
 

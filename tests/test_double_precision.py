@@ -107,7 +107,7 @@ def test_double_build_matches_oracle(name, mode, cuda, oracle):
     gi, gd = rng.standard_normal((H, W, 4)), rng.standard_normal((H, W))
     gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
                                         W, H, tw, th, m["per_pixel_sort"], ml, literal=False)
-    routes = [resume] + ([resume[:3] + (None,)] if resume[3] is not None else [])
+    routes = [resume] + ([resume[:3] + (None, None)] if resume[3] is not None or resume[4] is not None else [])
     for res in routes:
         out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                                  d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H,

@@ -48,7 +48,7 @@ def _forward_both(scene, tw, th, mode, cuda, oracle, thr=1 / 256):
 
 
 def _check_forward(name, want, got):
-    image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status, fragments) = got
+    image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status, fragments, hit_masks) = got
     assert int(status.item()) == 0
     np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
     np.testing.assert_array_equal(sorted_ids.cpu().numpy(), want["sorted_ids"])
@@ -120,7 +120,12 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
     # then the route that selects the fragments again is checked as well
     saved_order = resume[3] is not None
     assert saved_order == (bool(m["per_pixel_sort"]) and ml <= _C.MAX_SAVED_LAYERS)
-    routes = [("", resume)] + ([(" (re-selected)", resume[:3] + (None,))] if saved_order else [])
+    assert (resume[4] is not None) == (not m["per_pixel_sort"])  # tile order saves its hit masks
+    routes = [("", resume)]
+    if saved_order:
+        routes.append((" (re-selected)", resume[:3] + (None, None)))
+    if resume[4] is not None:
+        routes.append((" (inside tests repeated)", resume[:4] + (None,)))
     for route, res in routes:
         out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                                  d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H,

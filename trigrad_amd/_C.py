@@ -72,6 +72,9 @@ MAX_SAVED_LAYERS = 32  # TG_MAX_SAVED_LAYERS of the C header
 # blend order ((max_layers, H, W) int32) and the backward pass walks it in reverse instead of
 # selecting the fragments again.  False trades the memory for the re-selection.
 SAVE_BLEND_ORDER = True
+# Without per_pixel_sort the forward pass saves which list entries cover which pixel (one bit per pair it
+# looked at) and the backward pass reads that back instead of repeating the inside tests.
+SAVE_HIT_MASKS = True
 
 
 def scan_exclusive(counts, out=None, heads=None):
@@ -240,9 +243,9 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
     """Reference _C.render_forward (render.cu:713-763).
 
     -> (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume)
-    `resume` = (last, last_depth, status, fragments): what the backward pass needs
-    for its reverse traversal (fragments is None unless the blend order was saved),
-    plus the sort's status word.
+    `resume` = (last, last_depth, status, fragments, hit_masks): what the backward
+    pass needs for its reverse traversal (fragments / hit_masks are None unless the
+    blend order / the hit masks were saved), plus the sort's status word.
     """
     _need_cuda(vertices, indices, colors, opacities)
     bits = _bits(vertices)
@@ -295,14 +298,18 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             bary_transforms = cartesian_to_bary(vertices, indices)
 
         timer.start("rasterization")
+        hit_masks = None
+        if not per_pixel_sort and SAVE_HIT_MASKS:
+            words = int(lib.tg_hit_mask_words(K, width, height, tile_width, tile_height))
+            hit_masks = torch.empty((words,), dtype=torch.int64, device=dev)
         _lib.check(lib.tg_render_forward(
             _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
             width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
             _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
-            _stream(vertices)), "tg_render_forward", bits)
+            _ptr(hit_masks), _stream(vertices)), "tg_render_forward", bits)
         timings = timer.stop()
     return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
-            (last, last_depth, sort_status, fragments))
+            (last, last_depth, sort_status, fragments, hit_masks))
 
 
 def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
@@ -313,7 +320,7 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
     grad_depthmap may be None (no gradient reached the depth map)."""
     if resume is None:
         raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
-    last, last_depth, sort_status, fragments = resume
+    last, last_depth, sort_status, fragments, hit_masks = resume
     _need_cuda(grad_output, vertices)
     bits = _bits(vertices)
     lib = _lib.load(bits)
@@ -329,7 +336,7 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
         grad_colors = block[4 * V:7 * V].view(V, 3)
         grad_opacities = block[7 * V:]
         _lib.check(lib.tg_render_backward(
-            *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), width, height, tile_width, tile_height,
+            *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), _ptr(hit_masks), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
             _ptr(grad_opacities), _stream(vertices)), "tg_render_backward", bits)
     return grad_vertices, grad_colors, grad_opacities

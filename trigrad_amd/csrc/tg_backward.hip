@@ -32,6 +32,7 @@ struct BackwardArgs {
     const int32_t *last;
     const real *last_depth;
     const int32_t *fragments;  // saved by the forward pass, or null
+    const uint64_t *hit_masks; // saved by the tile-order forward pass, or null
     real *grad_vertices;
     real *grad_colors;
     real *grad_opacities;
@@ -386,39 +387,71 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     BackState st;
     if (p.valid) st = load_back_state(g, p);
 
-    for (int hi = tile_last; hi > 0; hi -= kBackBatch) {
-        const int lo = max(0, hi - kBackBatch);
-        const int nb = hi - lo;
+    // Batches are aligned to multiples of kBackBatch from the start of the list (the last one may be
+    // short), so that a batch is two whole words of the saved hit masks.
+    const bool saved_masks = g.hit_masks != nullptr;
+    const int64_t mask_slots = (int64_t)gridDim.z * blockDim.x, mask_slot = (int64_t)blockIdx.z * blockDim.x + tid;
+    for (int hi = (tile_last + kBackBatch - 1) / kBackBatch * kBackBatch; hi > 0; hi -= kBackBatch) {
+        const int lo = hi - kBackBatch;
+        const int nb = min(hi, tile_last) - lo;
         __syncthreads();  // every wave is done with the previous batch
         for (int e = tid; e < nb; e += blockDim.x) {
             gather_back(a, start + lo + e, s_rec[e]);
-            s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+            if (!saved_masks) s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
         }
         __syncthreads();
 
-        // 1. inside tests, only for the entries that can touch this wave's pixels
+        // 1. which entries cover which pixel: read back what the forward pass saved, or test again
+        //    (then only the entries that can touch this wave's pixels)
         const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
         if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
         ballots[lane] = 0;
         ballots[lane + kWave] = 0;
         wave_lds_sync();
         uint64_t m[2] = {0, 0};
+        if (saved_masks) {
+            const int64_t chunk = hit_mask_chunk(start, tile, lo);
 #pragma unroll
-        for (int wd = 0; wd < 2; wd++) {
-            uint64_t bits = 0;
-            uint64_t todo = wave_candidates(s_touch, 64 * wd, nb, wave);
-            while (todo) {
-                const int bit = __builtin_ctzll(todo);
-                todo &= todo - 1;
-                const BackRecord &r = s_rec[64 * wd + bit];
-                real b0, b1, b2;
-                bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                const bool hit = bary_inside(b0, b1, b2) && 64 * wd + bit < mine;
-                const uint64_t vote = __builtin_amdgcn_ballot_w64(hit);
-                if (hit) bits |= 1ull << bit;
-                if (lane == 0) ballots[64 * wd + bit] = vote;
+            for (int wd = 0; wd < 2; wd++) {
+                uint64_t bits = 0;
+                if (64 * wd < mine) {
+                    bits = g.hit_masks[(chunk + wd) * mask_slots + mask_slot];
+                    if (mine < 64 * wd + 64) bits &= (1ull << (mine - 64 * wd)) - 1;  // entries past my last one
+                }
+                m[wd] = bits;
+                // per-entry ballots = the transpose, for the entries any lane holds
+                uint32_t any_lo = (uint32_t)bits, any_hi = (uint32_t)(bits >> 32);
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) {
+                    any_lo |= __shfl_xor(any_lo, off, kWave);
+                    any_hi |= __shfl_xor(any_hi, off, kWave);
+                }
+                uint64_t todo = ((uint64_t)any_hi << 32) | any_lo;
+                while (todo) {
+                    const int bit = __builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    const uint64_t vote = __builtin_amdgcn_ballot_w64((bits >> bit) & 1);
+                    if (lane == 0) ballots[64 * wd + bit] = vote;
+                }
             }
-            m[wd] = bits;
+        } else {
+#pragma unroll
+            for (int wd = 0; wd < 2; wd++) {
+                uint64_t bits = 0;
+                uint64_t todo = wave_candidates(s_touch, 64 * wd, nb, wave);
+                while (todo) {
+                    const int bit = __builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    const BackRecord &r = s_rec[64 * wd + bit];
+                    real b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    const bool hit = bary_inside(b0, b1, b2) && 64 * wd + bit < mine;
+                    const uint64_t vote = __builtin_amdgcn_ballot_w64(hit);
+                    if (hit) bits |= 1ull << bit;
+                    if (lane == 0) ballots[64 * wd + bit] = vote;
+                }
+                m[wd] = bits;
+            }
         }
         wave_lds_sync();
 
@@ -755,7 +788,8 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
                                   const int32_t *indices, const real *colors, const real *opacities,
                                   const int32_t *sorted_ids, const int32_t *offsets, const real *bary, const real *image,
                                   const real *depthmap, const real *final_weights, const int32_t *ends, const int32_t *last,
-                                  const real *last_depth, const int32_t *fragments, int width, int height, int tile_w,
+                                  const real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width,
+                                  int height, int tile_w,
                                   int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers, real *grad_vertices,
                                   real *grad_colors, real *grad_opacities, void *stream) {
     if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
@@ -772,7 +806,7 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
     RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
     BackwardArgs g{(const real4 *)grad_image, grad_depthmap, (const real4 *)image, depthmap, final_weights, ends, last,
-                   last_depth, fragments, grad_vertices, grad_colors, grad_opacities};
+                   last_depth, fragments, per_pixel_sort ? nullptr : hit_masks, grad_vertices, grad_colors, grad_opacities};
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);

@@ -24,6 +24,7 @@ struct ForwardOut {
     int32_t *last;
     real *last_depth;
     int32_t *fragments;  // (max_layers, H, W): list positions, relative to the tile's start, in blend order; may be null
+    uint64_t *hit_masks; // tile order: which list entries cover which pixel, 64 entries per word (see hit_mask_chunk); may be null
 };
 
 __device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, real last_depth) {
@@ -70,6 +71,14 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         uint64_t m[kBatch / kWave];
         batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
         if (!running) m[0] = m[1] = m[2] = m[3] = 0;
+        if (out.hit_masks) {
+            // kept for the backward pass, which then has no inside test to repeat
+            const int64_t chunk = hit_mask_chunk(start, tile, batch - start);
+            const int64_t slots = (int64_t)gridDim.z * blockDim.x, slot = (int64_t)blockIdx.z * blockDim.x + tid;
+#pragma unroll
+            for (int wd = 0; wd < kBatch / kWave; wd++)
+                if (wd * kWave < nb) out.hit_masks[(chunk + wd) * slots + slot] = m[wd];
+        }
         // 2. every lane composites its own hits in list order, so the blend arithmetic
         //    runs with as many lanes busy as there are pixels with a fragment left
         while (true) {
@@ -280,11 +289,18 @@ int check_raster_args(const char *fn, int width, int height, int tile_w, int til
 
 using namespace tg;
 
+extern "C" size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int tile_w, int tile_h) {
+    if (n_keys < 0 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0 || tile_w * tile_h > kMaxTilePixels) return 0;
+    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
+    const int64_t tiles = (int64_t)tl.grid.x * tl.grid.y;
+    return (size_t)((n_keys / kWave + tiles + 1) * (int64_t)tl.grid.z * tl.threads);
+}
+
 extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, const real *colors, const real *opacities,
                                  const int32_t *sorted_ids, const int32_t *offsets, const real *bary, int width, int height,
                                  int tile_w, int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers,
                                  real *image, real *depthmap, real *final_weights, int32_t *ends, int32_t *last,
-                                 real *last_depth, int32_t *fragments, void *stream) {
+                                 real *last_depth, int32_t *fragments, uint64_t *hit_masks, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
         set_error("tg_render_forward: null pointer");
@@ -300,7 +316,7 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         set_error("tg_render_forward: fragments are saved only with per_pixel_sort and max_layers <= %d", TG_MAX_SAVED_LAYERS);
         return TG_E_ARG;
     }
-    ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments};
+    ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments, per_pixel_sort ? nullptr : hit_masks};
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads(128) : kTileThreads);
     const dim3 grid = tl.grid;
     const int n_threads = tl.threads;

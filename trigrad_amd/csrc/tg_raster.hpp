@@ -110,6 +110,15 @@ __device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRe
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
 }
 
+// Saved hit masks (tile order): word (chunk * slots + slot) holds, for the pixel
+// in thread slot `slot` of its tile, which of 64 consecutive list entries cover
+// it.  The chunks of a tile whose list starts at `start` are numbered from
+// start / 64 + tile: consecutive tiles never share a chunk, and
+// n_keys / 64 + n_tiles + 1 chunks hold every list.
+__device__ __forceinline__ int64_t hit_mask_chunk(int start, int tile, int relative_position) {
+    return (int64_t)(start >> 6) + tile + (relative_position >> 6);
+}
+
 // Front-to-back compositing state of one pixel (render.cu:564-574).
 struct PixelState {
     real alpha = 1.0f, c0 = 0.0f, c1 = 0.0f, c2 = 0.0f, depth = 0.0f, weight = 0.0f;

@@ -53,14 +53,15 @@ class Renderer(Function):
             (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume) = _C.render_forward(
                 vertices, indices, colors, opacities, width, height, tile_width, tile_height, early_stopping_threshold,
                 not record_timing, per_pixel_sort, max_layers)
-            last, last_depth, sort_status, fragments = resume
+            last, last_depth, sort_status, fragments, hit_masks = resume
             if record_timing and int(sort_status.item()) != 0:
                 raise RuntimeError("tg_sort_pairs_u64_u32: look-back wait timed out")
-            # private to this Function: where the reverse traversal starts, and (per-pixel order,
-            # max_layers <= 32) the blend order itself
-            extras = [t for t in (last_depth, fragments) if t is not None]
+            # private to this Function: where the reverse traversal starts, and the blend order (per-pixel
+            # order, max_layers <= 32) or the hit masks (tile order)
+            extras = [t for t in (last_depth, fragments, hit_masks) if t is not None]
             ctx.has_last_depth = last_depth is not None
             ctx.has_fragments = fragments is not None
+            ctx.has_hit_masks = hit_masks is not None
             saved = [vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, image, depthmap, final_weights,
                      ends, last, sort_status]
             ctx.save_for_backward(*saved, *extras)
@@ -80,12 +81,13 @@ class Renderer(Function):
             extras = list(saved[13:])
             last_depth = extras.pop(0) if ctx.has_last_depth else None
             fragments = extras.pop(0) if ctx.has_fragments else None
+            hit_masks = extras.pop(0) if ctx.has_hit_masks else None
             width, height, tile_width, tile_height, threshold, per_pixel_sort, max_layers = ctx.render_args
             if grad_image is None:
                 grad_image = torch.zeros_like(saved[7])
             grad_vertices, grad_colors, grad_opacities = _C.render_backward(
                 grad_image, grad_depthmap, *saved[:11], width, height, tile_width, tile_height, threshold, per_pixel_sort,
-                max_layers, resume=(last, last_depth, sort_status, fragments))
+                max_layers, resume=(last, last_depth, sort_status, fragments, hit_masks))
         # one slot per forward argument (wrapper.py:99-112)
         return (grad_vertices, None, grad_colors, grad_opacities, None, None, None, None, None, None, None, None)
 
