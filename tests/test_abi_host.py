@@ -54,7 +54,7 @@ def test_host_side_helpers_and_argument_rejection(bits):
     assert b"tile_w*tile_h" in lib.tg_last_error()
     assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 9)) == -1
     assert b"max_layers" in lib.tg_last_error()
-    assert lib.tg_render_backward(*([None] * 17), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, None) == -1
+    assert lib.tg_render_backward(*([None] * 17), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, 4, 3, 1, None) == -1
     assert lib.tg_hit_mask_words(6400, 64, 64, 16, 16) == (100 + 16 + 1) * 256
     with pytest.raises(RuntimeError, match="tg_bin_count failed with code -1"):
         _lib.check(lib.tg_bin_count(None, 0, None, -1, 64, 64, 16, 16, None, None), "tg_bin_count", bits)

@@ -329,16 +329,28 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
         tensors = [None if t is None else t.contiguous()
                    for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
                              bary_transforms, image, depthmap, final_weights, ends, last)]
-        # one zero fill for the three gradients: (V,4) | (V,3) | (V,) views of one block
+        # one zero fill for the three gradients.  Tile order: (V,4) | (V,3) | (V,) views of one block.  Per-pixel
+        # order issues five times as many atomics; there the eight gradients of a vertex share a 32-byte
+        # sector of a (V,8) block while the kernel runs, and the three arrays are copied out afterwards.
         V = vertices.shape[0]
         block = torch.zeros((8 * V,), dtype=vertices.dtype, device=dev)
-        grad_vertices = block[:4 * V].view(V, 4)
-        grad_colors = block[4 * V:7 * V].view(V, 3)
-        grad_opacities = block[7 * V:]
+        interleaved = bool(per_pixel_sort)
+        if interleaved:
+            b8 = block.view(V, 8)
+            grad_vertices, grad_colors, grad_opacities = b8[:, 0:4], b8[:, 4:7], b8[:, 7]
+            strides = (8, 8, 8)
+        else:
+            grad_vertices = block[:4 * V].view(V, 4)
+            grad_colors = block[4 * V:7 * V].view(V, 3)
+            grad_opacities = block[7 * V:]
+            strides = (4, 3, 1)
         _lib.check(lib.tg_render_backward(
             *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), _ptr(hit_masks), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
-            _ptr(grad_opacities), _stream(vertices)), "tg_render_backward", bits)
+            _ptr(grad_opacities), *strides, _stream(vertices)), "tg_render_backward", bits)
+        if interleaved:
+            grad_vertices, grad_colors, grad_opacities = (grad_vertices.contiguous(), grad_colors.contiguous(),
+                                                          grad_opacities.contiguous())
     return grad_vertices, grad_colors, grad_opacities
 
 

@@ -36,6 +36,7 @@ struct BackwardArgs {
     real *grad_vertices;
     real *grad_colors;
     real *grad_opacities;
+    int vertex_stride, color_stride, opacity_stride;  // scalars from one vertex to the next in the three arrays
 };
 
 // process_backward's inputs for one list entry.
@@ -259,10 +260,10 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
 }
 
 __device__ __forceinline__ real *term_address(const BackwardArgs &g, int vertex_id, int c) {
-    if (c < 2) return g.grad_vertices + 4 * (int64_t)vertex_id + c;
-    if (c == 2) return g.grad_vertices + 4 * (int64_t)vertex_id + 3;
-    if (c < 6) return g.grad_colors + 3 * (int64_t)vertex_id + (c - 3);
-    return g.grad_opacities + vertex_id;
+    if (c < 2) return g.grad_vertices + g.vertex_stride * (int64_t)vertex_id + c;
+    if (c == 2) return g.grad_vertices + g.vertex_stride * (int64_t)vertex_id + 3;
+    if (c < 6) return g.grad_colors + g.color_stride * (int64_t)vertex_id + (c - 3);
+    return g.grad_opacities + g.opacity_stride * (int64_t)vertex_id;
 }
 
 __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, const PixelCoord &p) {
@@ -791,12 +792,17 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
                                   const real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width,
                                   int height, int tile_w,
                                   int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers, real *grad_vertices,
-                                  real *grad_colors, real *grad_opacities, void *stream) {
+                                  real *grad_colors, real *grad_opacities, int vertex_stride, int color_stride,
+                                  int opacity_stride, void *stream) {
     if (int e = check_raster_args("tg_render_backward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!grad_image || !vertices || !indices || !colors || !opacities || !offsets || !bary || !image ||
         !depthmap || !final_weights || !ends || !last || !grad_vertices || !grad_colors || !grad_opacities ||
         (per_pixel_sort && !last_depth && !fragments)) {
         set_error("tg_render_backward: null pointer");
+        return TG_E_ARG;
+    }
+    if (vertex_stride < 4 || color_stride < 3 || opacity_stride < 1) {
+        set_error("tg_render_backward: gradient strides must be at least 4, 3 and 1");
         return TG_E_ARG;
     }
     if (((uintptr_t)vertices & 15) || ((uintptr_t)image & 15) || ((uintptr_t)grad_image & 15)) {
@@ -806,7 +812,8 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
     RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
     BackwardArgs g{(const real4 *)grad_image, grad_depthmap, (const real4 *)image, depthmap, final_weights, ends, last,
-                   last_depth, fragments, per_pixel_sort ? nullptr : hit_masks, grad_vertices, grad_colors, grad_opacities};
+                   last_depth, fragments, per_pixel_sort ? nullptr : hit_masks, grad_vertices, grad_colors, grad_opacities,
+                   vertex_stride, color_stride, opacity_stride};
     hipStream_t s = (hipStream_t)stream;
     if (!per_pixel_sort) {
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
