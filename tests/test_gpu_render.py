@@ -206,6 +206,42 @@ def test_loss_on_depth_only(cuda, oracle):
     assert float(v.grad.abs().max()) > 0
 
 
+@pytest.mark.parametrize("mode", ["A_default", "B_unlimited"])
+def test_repeatable_and_stream_ordered(mode, cuda):
+    """Two calls give bit-identical images and lists (only the gradient sums depend on the order of atomics), and a
+    call on a side stream, ordered after the inputs' producer, gives the same result as on the default stream."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import scenes as S
+    if mode not in MODES:
+        pytest.skip("mode table changed")
+    kw = dict(per_pixel_sort=MODES[mode]["per_pixel_sort"], max_layers=MODES[mode]["max_layers"])
+    scene = S.random_soup(2500, 200, 160, seed=31, sigma_px=10.0, varying_w=True)
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+
+    def run():
+        v = d["vertices"].clone().requires_grad_()
+        c = d["colors"].clone().requires_grad_()
+        o = d["opacities"].clone().requires_grad_()
+        image, depthmap = trigrad_amd.render(v, d["indices"], c, o, W, H, **kw)
+        (image.square().sum() + torch.where(torch.isfinite(depthmap), depthmap, torch.zeros_like(depthmap)).sum()).backward()
+        return image.detach(), depthmap.detach(), v.grad, c.grad, o.grad
+
+    first = run()
+    second = run()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        third = run()
+    side.synchronize()
+    for other in (second, third):
+        assert torch.equal(first[0], other[0]) and torch.equal(first[1], other[1])
+        for a, b in zip(first[2:], other[2:]):
+            scale = float(a.abs().max())
+            assert float((a - b).abs().max()) <= 1e-5 * scale + 1e-6
+
+
 def test_record_timing_and_empty_scene(cuda):
     import torch
     import trigrad_amd
