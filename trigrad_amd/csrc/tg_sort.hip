@@ -78,9 +78,13 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
 
 __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, int passes,
                                                                       uint32_t *__restrict__ partials) {
-    __shared__ uint32_t s_hist[kMaxPasses][kRadix];
+    // one set of counters per wave: the upper passes see few distinct digits (the tile bits), and LDS
+    // atomics to one address serialise
+    __shared__ uint32_t s_hist_wave[kSortWaves][kMaxPasses][kRadix];
     const int tid = threadIdx.x;
-    for (int p = 0; p < passes; p++) s_hist[p][tid] = 0;
+    uint32_t (*s_hist)[kRadix] = s_hist_wave[tid / kWave];
+    for (int w = 0; w < kSortWaves; w++)
+        for (int p = 0; p < passes; p++) s_hist_wave[w][p][tid] = 0;
     __syncthreads();
     const int64_t stride = (int64_t)gridDim.x * kSortThreads * 4;
     for (int64_t i = (int64_t)blockIdx.x * kSortThreads * 4 + tid; i < n; i += stride) {
@@ -94,7 +98,12 @@ __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint
     }
     __syncthreads();
     uint32_t *out = partials + (size_t)blockIdx.x * kMaxPasses * kRadix;
-    for (int p = 0; p < passes; p++) out[p * kRadix + tid] = s_hist[p][tid];
+    for (int p = 0; p < passes; p++) {
+        uint32_t sum = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; w++) sum += s_hist_wave[w][p][tid];
+        out[p * kRadix + tid] = sum;
+    }
 }
 
 // One workgroup per pass: digit totals over all partials (four groups of 256
