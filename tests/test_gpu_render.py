@@ -139,6 +139,15 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
                          GRAD_ATOL + 2e-6 * scale)
             assert np.array_equal(np.isnan(g), np.isnan(w))
         assert float(out[0][:, 2].abs().max()) == 0.0  # z never receives a gradient (render.cu:531-533)
+    if name == "soup_shared" and with_depth:
+        # the three layouts of the gradient arrays the kernels know: dense, one (V,8) block, run-time strides
+        for strides in ((4, 3, 1), (8, 8, 8), (6, 5, 2)):
+            alt = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
+                                     d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W,
+                                     H, tw, th, 1 / 256, m["per_pixel_sort"], ml, resume=resume, grad_strides=strides)
+            for a, b in zip(alt, out):
+                assert a.is_contiguous() and a.shape == b.shape
+                assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max()) + 1e-6
 
 
 def test_default_mode_literal_and_policy_agree(oracle):

@@ -314,10 +314,12 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
 
 def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
                     image, depthmap, final_weights, ends, width, height, tile_width, tile_height, early_stopping_threshold,
-                    per_pixel_sort, max_layers, resume=None):
+                    per_pixel_sort, max_layers, resume=None, grad_strides=None):
     """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities).
 
-    grad_depthmap may be None (no gradient reached the depth map)."""
+    grad_depthmap may be None (no gradient reached the depth map).  grad_strides (scalars per vertex in the
+    three arrays the kernel accumulates into) defaults to dense arrays in tile order and to one (V,8) block
+    with per_pixel_sort; the returned tensors are dense either way."""
     if resume is None:
         raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
     last, last_depth, sort_status, fragments, hit_masks = resume
@@ -333,22 +335,25 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
         # order issues five times as many atomics; there the eight gradients of a vertex share a 32-byte
         # sector of a (V,8) block while the kernel runs, and the three arrays are copied out afterwards.
         V = vertices.shape[0]
-        block = torch.zeros((8 * V,), dtype=vertices.dtype, device=dev)
-        interleaved = bool(per_pixel_sort)
-        if interleaved:
-            b8 = block.view(V, 8)
-            grad_vertices, grad_colors, grad_opacities = b8[:, 0:4], b8[:, 4:7], b8[:, 7]
-            strides = (8, 8, 8)
-        else:
+        strides = tuple(grad_strides) if grad_strides is not None else ((8, 8, 8) if per_pixel_sort else (4, 3, 1))
+        if strides == (4, 3, 1):
+            block = torch.zeros((8 * V,), dtype=vertices.dtype, device=dev)
             grad_vertices = block[:4 * V].view(V, 4)
             grad_colors = block[4 * V:7 * V].view(V, 3)
             grad_opacities = block[7 * V:]
-            strides = (4, 3, 1)
+        elif strides == (8, 8, 8):
+            b8 = torch.zeros((V, 8), dtype=vertices.dtype, device=dev)
+            grad_vertices, grad_colors, grad_opacities = b8[:, 0:4], b8[:, 4:7], b8[:, 7]
+        else:
+            sv, sc, so = strides
+            grad_vertices = torch.zeros((V, sv), dtype=vertices.dtype, device=dev)[:, :4]
+            grad_colors = torch.zeros((V, sc), dtype=vertices.dtype, device=dev)[:, :3]
+            grad_opacities = torch.zeros((V, so), dtype=vertices.dtype, device=dev)[:, 0]
         _lib.check(lib.tg_render_backward(
             *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), _ptr(hit_masks), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
             _ptr(grad_opacities), *strides, _stream(vertices)), "tg_render_backward", bits)
-        if interleaved:
+        if strides != (4, 3, 1):
             grad_vertices, grad_colors, grad_opacities = (grad_vertices.contiguous(), grad_colors.contiguous(),
                                                           grad_opacities.contiguous())
     return grad_vertices, grad_colors, grad_opacities

@@ -259,11 +259,20 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
     fragment_terms(f, r, b0, b1, b2, px, py, out);
 }
 
+// Layout of the three gradient arrays, a template parameter of the kernels so that the two layouts
+// in use address with constants: dense (4, 3, 1 scalars per vertex), one (V,8) block (8, 8, 8), or
+// the strides given at run time.
+enum GradLayout { kGradDense = 0, kGradBlock8 = 1, kGradStrided = 2 };
+
+template <int kLayout>
 __device__ __forceinline__ real *term_address(const BackwardArgs &g, int vertex_id, int c) {
-    if (c < 2) return g.grad_vertices + g.vertex_stride * (int64_t)vertex_id + c;
-    if (c == 2) return g.grad_vertices + g.vertex_stride * (int64_t)vertex_id + 3;
-    if (c < 6) return g.grad_colors + g.color_stride * (int64_t)vertex_id + (c - 3);
-    return g.grad_opacities + g.opacity_stride * (int64_t)vertex_id;
+    const int sv = kLayout == kGradDense ? 4 : kLayout == kGradBlock8 ? 8 : g.vertex_stride;
+    const int sc = kLayout == kGradDense ? 3 : kLayout == kGradBlock8 ? 8 : g.color_stride;
+    const int so = kLayout == kGradDense ? 1 : kLayout == kGradBlock8 ? 8 : g.opacity_stride;
+    if (c < 2) return g.grad_vertices + sv * (int64_t)vertex_id + c;
+    if (c == 2) return g.grad_vertices + sv * (int64_t)vertex_id + 3;
+    if (c < 6) return g.grad_colors + sc * (int64_t)vertex_id + (c - 3);
+    return g.grad_opacities + so * (int64_t)vertex_id;
 }
 
 __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, const PixelCoord &p) {
@@ -353,6 +362,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 //      evaluates the 21 gradient terms of its hit and writes them to a term
 //      matrix; three groups of 21 lanes add up the runs of equal entry and issue
 //      one global floating-point atomic per run and term.
+template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ BackRecord s_rec[kBackBatch];
     __shared__ uint64_t s_ballot[kMaxWaves][kBackBatch];
@@ -533,7 +543,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 if (group < 3 && c0 < c1)
                     sum_runs(terms + q * kTermStride, c0, c1,
                              [&](int c) { return int_of_real(seeds[5][s0 + c]) & 0xff; },
-                             [&](int entry, real sum) { unsafeAtomicAdd(term_address(g, s_rec[entry].id[q / 7], q % 7), sum); });
+                             [&](int entry, real sum) { unsafeAtomicAdd(term_address<kLayout>(g, s_rec[entry].id[q / 7], q % 7), sum); });
                 wave_lds_sync();
             }
         }
@@ -561,6 +571,7 @@ __device__ __forceinline__ void topk_insert_desc(const TopK &tk, int cap, int &n
     if (n < cap) n++;
 }
 
+template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(RasterArgs a, BackwardArgs g) {
     extern __shared__ __align__(16) unsigned char s_dyn[];
     const int n_threads = blockDim.x;
@@ -640,7 +651,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
                 } else {
 #pragma unroll
                     for (int q = 0; q < kTerms; q++)
-                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address<kLayout>(g, r.id[q / 7], q % 7), term[q]);
                 }
             }
             if (found < cap) {
@@ -659,7 +670,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 #pragma unroll
         for (int q = 0; q < kTerms; q++) {
             const real v = s_acc[e * kTerms + q];
-            if (v != 0.0f) unsafeAtomicAdd(term_address(g, id[q / 7], q % 7), v);
+            if (v != 0.0f) unsafeAtomicAdd(term_address<kLayout>(g, id[q / 7], q % 7), v);
         }
     }
 }
@@ -680,6 +691,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 constexpr int kSavedWindow = 256;
 constexpr int kSavedStride = kBackReals + 4;  // 33 scalars, 3 vertex ids; odd
 
+template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ real s_rows[kSavedWindow * kSavedStride];
     __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
@@ -741,7 +753,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
                 if (!staged) {
 #pragma unroll
                     for (int q = 0; q < kTerms; q++)
-                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address(g, r.id[q / 7], q % 7), term[q]);
+                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address<kLayout>(g, r.id[q / 7], q % 7), term[q]);
                 }
             }
             // slots: lanes with the same entry next to each other, groups in order of their lowest lane
@@ -772,7 +784,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
             const int c0 = group * per, c1 = min(c0 + per, n_slots);
             if (group < 3 && c0 < c1)
                 sum_runs(terms + q * kTermStride, c0, c1, [&](int c) { return tags[c]; }, [&](int entry, real sum) {
-                    unsafeAtomicAdd(term_address(g, int_of_real(s_rows[entry * kSavedStride + kBackReals + q / 7]), q % 7), sum);
+                    unsafeAtomicAdd(term_address<kLayout>(g, int_of_real(s_rows[entry * kSavedStride + kBackReals + q / 7]), q % 7), sum);
                 });
             wave_lds_sync();
         }
@@ -815,9 +827,18 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
                    last_depth, fragments, per_pixel_sort ? nullptr : hit_masks, grad_vertices, grad_colors, grad_opacities,
                    vertex_stride, color_stride, opacity_stride};
     hipStream_t s = (hipStream_t)stream;
+    const int layout = (vertex_stride == 4 && color_stride == 3 && opacity_stride == 1)   ? kGradDense
+                       : (vertex_stride == 8 && color_stride == 8 && opacity_stride == 8) ? kGradBlock8
+                                                                                          : kGradStrided;
+#define TG_LAUNCH_BACKWARD(kernel, grid, block, lds_bytes)                                                  \
+    do {                                                                                                    \
+        if (layout == kGradDense) TG_LAUNCH_AS(#kernel, kernel<kGradDense>, grid, block, lds_bytes, s, a, g);   \
+        else if (layout == kGradBlock8) TG_LAUNCH_AS(#kernel, kernel<kGradBlock8>, grid, block, lds_bytes, s, a, g); \
+        else TG_LAUNCH_AS(#kernel, kernel<kGradStrided>, grid, block, lds_bytes, s, a, g);                      \
+    } while (0)
     if (!per_pixel_sort) {
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
-        TG_LAUNCH(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
+        TG_LAUNCH_BACKWARD(backward_tile_order_kernel, tl.grid, dim3(tl.threads), 0);
         return check_launch("backward_tile_order_kernel");
     }
     if (fragments) {
@@ -826,13 +847,19 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
             return TG_E_ARG;
         }
         const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
-        TG_LAUNCH(backward_saved_order_kernel, tl.grid, dim3(tl.threads), 0, s, a, g);
+        TG_LAUNCH_BACKWARD(backward_saved_order_kernel, tl.grid, dim3(tl.threads), 0);
         return check_launch("backward_saved_order_kernel");
     }
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads(kTileThreads));
     const size_t lds = backward_pixel_order_lds_bytes(tl.threads);
     static size_t lds_reserved = 0;
-    if (int e = reserve_lds("tg_render_backward", (const void *)backward_pixel_order_kernel, lds, &lds_reserved)) return e;
-    TG_LAUNCH(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds, s, a, g);
+    for (const void *kernel : {(const void *)backward_pixel_order_kernel<kGradDense>, (const void *)backward_pixel_order_kernel<kGradBlock8>,
+                               (const void *)backward_pixel_order_kernel<kGradStrided>}) {
+        size_t none = 0;
+        if (int e = reserve_lds("tg_render_backward", kernel, lds, lds <= lds_reserved ? &lds_reserved : &none)) return e;
+    }
+    if (lds > lds_reserved) lds_reserved = lds;
+    TG_LAUNCH_BACKWARD(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds);
     return check_launch("backward_pixel_order_kernel");
+#undef TG_LAUNCH_BACKWARD
 }

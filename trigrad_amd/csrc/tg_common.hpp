@@ -51,11 +51,12 @@ struct ProfileScope {
     int slot;
     hipStream_t stream;
 };
-#define TG_LAUNCH(kernel, grid, block, lds, stream, ...)               \
+#define TG_LAUNCH_AS(name, kernel, grid, block, lds, stream, ...)       \
     do {                                                               \
-        tg::ProfileScope tg_profile_scope(#kernel, stream);            \
+        tg::ProfileScope tg_profile_scope(name, stream);               \
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__); \
     } while (0)
+#define TG_LAUNCH(kernel, grid, block, lds, stream, ...) TG_LAUNCH_AS(#kernel, kernel, grid, block, lds, stream, __VA_ARGS__)
 
 // Workgroups of `kernel` that can be resident on the current device at once
 // (0 if unknown).  A grid that is no larger needs no ticket to number its
