@@ -169,6 +169,12 @@ def main():
         other = "A" if args.mode == "B" else "B"
         extra[f"mode_{other}_fwd_bwd_fps"] = 1000.0 / timed(lambda: step(other), max(3, args.steps // 2), 1)
         extra[f"mode_{other}_forward_only_fps"] = 1000.0 / timed(lambda: step(other, backward=False), max(3, args.steps // 2), 1)
+        # what a plain device copy reaches on this box (256 MiB read + 256 MiB written), for scale
+        src = torch.empty((64 << 20,), dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        t_copy = timed(lambda: dst.copy_(src), 10, 2)
+        extra["device_copy_GBps"] = 2.0 * src.numel() * 4 / (t_copy / 1000.0) / 1e9
+        del src, dst
         # standalone sort at the scale the metric names
         n = args.sort_keys
         keys_np, vals_np = scenes.sort_keys(n, T, seed=0)
@@ -187,6 +193,18 @@ def main():
         t_sort = timed(sort_once, 10, 2) - timed(copy_only, 10, 2)
         extra["sort_standalone"] = {"keys": n, "ms": t_sort, "Gkeys_per_s": n / (t_sort / 1000.0) / 1e9,
                                     "GBps": (8.0 + 24.0 * passes) * n / (t_sort / 1000.0) / 1e9}
+        # the sweep kernel alone at this size, from the library's events: 24 bytes per pair and launch
+        _C.profile_enable(True)
+        _C.profile_report()
+        for _ in range(5):
+            sort_once()
+        torch.cuda.synchronize()
+        big = _C.profile_report()
+        _C.profile_enable(False)
+        launches, total_ms = big["sort_sweep_kernel"]
+        sweep_us = total_ms / launches * 1000.0
+        extra["sort_standalone"]["sweep_kernel"] = {"avg_launch_us": sweep_us, "GBps": 24.0 * n / (sweep_us * 1e-6) / 1e9,
+                                                    "frac_of_hbm_peak": 24.0 * n / (sweep_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
     out["extra"] = extra
 
     if not args.no_cpu_baseline:
