@@ -385,18 +385,18 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     real (*seeds)[kWaveSlots] = s_seed[wave];
     real *terms = s_term[wave];
 
+    // the pixel's loads are issued before the barriers below, which then cover their latency
+    const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
+    BackState st;
+    if (p.valid) st = load_back_state(g, p);
     if (tid == 0) s_last = 0;
     s_px[tid] = p.px;
     s_py[tid] = p.py;
-    publish_wave_rect(p, s_rects);
+    if (!g.hit_masks) publish_wave_rect(p, s_rects);  // only the repeated inside tests cull by wave rectangle
     __syncthreads();
-    const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
     if (my_last > 0) atomicMax(&s_last, my_last);
     __syncthreads();
     const int tile_last = s_last;
-
-    BackState st;
-    if (p.valid) st = load_back_state(g, p);
 
     // Batches are aligned to multiples of kBackBatch from the start of the list (the last one may be
     // short), so that a batch is two whole words of the saved hit masks.
