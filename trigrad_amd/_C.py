@@ -37,6 +37,22 @@ def _stream(t):
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
+class _on_device:
+    """`with _on_device(dev)` that costs nothing when dev is already current (the stages of a frame nest)."""
+
+    def __init__(self, device):
+        self.guard = None if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
 def _need_cuda(*tensors):
     for t in tensors:
         if t.device.type != "cuda":
@@ -60,7 +76,7 @@ def bin_count(vertices, indices, width, height, tile_width, tile_height):
     lib = _lib.load(_bits(vertices))
     M = indices.shape[0]
     counts = torch.empty((M,), dtype=torch.int32, device=vertices.device)
-    with torch.cuda.device(vertices.device):
+    with _on_device(vertices.device):
         _lib.check(lib.tg_bin_count(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
                                     _ptr(counts), _stream(vertices)), "tg_bin_count", _bits(vertices))
     return counts
@@ -94,7 +110,7 @@ def scan_exclusive(counts, out=None, heads=None):
     total, status = pair[:1], pair[1:]
     ws_bytes = int(lib.tg_scan_workspace_bytes(n))
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.tg_scan_exclusive_u32(_ptr(counts), _ptr(out), n, _ptr(total), _ptr(ws), ws_bytes, _ptr(status), OWNER_STRIDE,
                                              0 if heads is None else heads.numel(), _ptr(heads), _stream(counts)),
                    "tg_scan_exclusive_u32")
@@ -115,7 +131,7 @@ def bin_emit(vertices, indices, tri_offsets, n_keys, width, height, tile_width, 
     dev = vertices.device
     keys = torch.empty((n_keys * (2 if _bits(vertices) == 64 else 1),), dtype=torch.int64, device=dev)
     payload = torch.empty((n_keys,), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.tg_bin_emit(_ptr(vertices), vertices.shape[0], _ptr(indices), indices.shape[0], width, height, tile_width,
                                    tile_height, _ptr(tri_offsets), n_keys, _ptr(heads), 0 if heads is None else heads.numel(),
                                    _ptr(keys), _ptr(payload), _stream(vertices)), "tg_bin_emit", _bits(vertices))
@@ -138,7 +154,7 @@ def sort_pairs(keys, values, end_bit=64):
     ws_bytes = int(lib.tg_sort_workspace_bytes(n))
     ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
     in_alt = C.c_int(0)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(lib.tg_sort_pairs_u64_u32(_ptr(keys), _ptr(values), _ptr(keys_alt), _ptr(values_alt), n, end_bit, _ptr(ws),
                                              ws_bytes, _ptr(status), C.byref(in_alt), _stream(keys)), "tg_sort_pairs_u64_u32")
     if in_alt.value:
@@ -151,7 +167,7 @@ def tile_ranges(sorted_keys, n_tiles):
     _need_cuda(sorted_keys)
     lib = _lib.load()
     offsets = torch.empty((n_tiles + 1,), dtype=torch.int32, device=sorted_keys.device)
-    with torch.cuda.device(sorted_keys.device):
+    with _on_device(sorted_keys.device):
         _lib.check(lib.tg_tile_ranges(_ptr(sorted_keys), sorted_keys.numel(), n_tiles, _ptr(offsets), _stream(sorted_keys)),
                    "tg_tile_ranges")
     return offsets
@@ -165,7 +181,7 @@ def cartesian_to_bary(vertices, indices):
     indices = indices.contiguous()
     M = indices.shape[0]
     out = torch.empty((M, 3, 3), dtype=vertices.dtype, device=vertices.device)
-    with torch.cuda.device(vertices.device):
+    with _on_device(vertices.device):
         _lib.check(lib.tg_bary(_ptr(vertices), vertices.shape[0], _ptr(indices), M, _ptr(out), _stream(vertices)), "tg_bary", _bits(vertices))
     return out
 
@@ -253,7 +269,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
     real = vertices.dtype
     timer = _StageTimer(disable_timing)
     dev = vertices.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         timer.start("init")
         vertices = vertices.contiguous()
         indices = indices.contiguous()
@@ -327,7 +343,7 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
     bits = _bits(vertices)
     lib = _lib.load(bits)
     dev = vertices.device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         tensors = [None if t is None else t.contiguous()
                    for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
                              bary_transforms, image, depthmap, final_weights, ends, last)]
