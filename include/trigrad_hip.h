@@ -138,6 +138,24 @@ int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int
 int tg_bary(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, tg_real *out,
             void *stream);
 
+/* ---- depth bounds of the lists (optional) ------------------------------------- */
+
+/* bounds (tg_list_bound_words() scalars): for every tile and every 256 entries
+ * of its list a lower bound of the per-pixel depth (render.cu:404) of the
+ * entries from there to far_start[tile]; far_start (n_tiles int32): the list
+ * position from which on the entries have the sort key 1e30 (empty clipped
+ * polygon, render.cu:259: they sit at the end whatever their depth).  With
+ * both, the per_pixel_sort selection of tg_render_forward
+ * (select_next_k_in_tile, render.cu:375-415, which always scans the whole list)
+ * skips from the point where every pixel's 32 candidates are nearer than
+ * anything the bounds cover to far_start: same result, and lists of thousands
+ * of entries are not scanned to the end.  triangle_low: n_triangles scalars of
+ * working memory (every triangle's own bound). */
+size_t tg_list_bound_words(int64_t n_keys, int n_tiles);
+int tg_list_bounds(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles,
+                   const uint64_t *sorted_keys, const int32_t *sorted_ids, const int32_t *offsets, int n_tiles,
+                   tg_real *triangle_low, tg_real *bounds, int32_t *far_start, void *stream);
+
 /* ---- (4) forward blend ------------------------------------------------------ */
 
 /* One workgroup per tile composites the tile's sorted list.  Replaces
@@ -158,13 +176,15 @@ int tg_bary(const tg_real *vertices, int32_t n_vertices, const int32_t *indices,
  * the kernel also writes, for every pixel and every 64 consecutive entries of
  * its tile's list that it looked at, which of them cover the pixel;
  * tg_render_backward then reads them back instead of repeating the inside tests.
+ * batch_bounds, far_start: tg_list_bounds' outputs, or NULL (used with per_pixel_sort only).
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
 size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int tile_w, int tile_h);
 int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_real *colors, const tg_real *opacities,
                       const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, int width, int height,
                       int tile_w, int tile_h, tg_real early_stopping_threshold, int per_pixel_sort, int max_layers,
                       tg_real *image, tg_real *depthmap, tg_real *final_weights, int32_t *ends, int32_t *last,
-                      tg_real *last_depth, int32_t *fragments, uint64_t *hit_masks, void *stream);
+                      tg_real *last_depth, int32_t *fragments, uint64_t *hit_masks,
+                      const tg_real *batch_bounds, const int32_t *far_start, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
 

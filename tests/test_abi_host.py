@@ -50,12 +50,14 @@ def test_host_side_helpers_and_argument_rejection(bits):
     res = C.c_int(7)
     assert lib.tg_sort_pairs_u64_u32(None, None, None, None, 1 << 31, 64, None, 0, None, C.byref(res), None) == -1
     assert lib.tg_tile_ranges(None, 5, 10, None, None) == -1
-    assert lib.tg_render_forward(*([None] * 7), 64, 64, 64, 32, 0.0, 0, 1, *([None] * 9)) == -1
+    assert lib.tg_render_forward(*([None] * 7), 64, 64, 64, 32, 0.0, 0, 1, *([None] * 11)) == -1
     assert b"tile_w*tile_h" in lib.tg_last_error()
-    assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 9)) == -1
+    assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 11)) == -1
     assert b"max_layers" in lib.tg_last_error()
     assert lib.tg_render_backward(*([None] * 17), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, 4, 3, 1, None) == -1
     assert lib.tg_hit_mask_words(6400, 64, 64, 16, 16) == (100 + 16 + 1) * 256
+    assert lib.tg_list_bound_words(6400, 16) == 25 + 16 + 1
+    assert lib.tg_list_bounds(None, 0, None, 0, None, None, None, 0, None, None, None, None) == -1
     with pytest.raises(RuntimeError, match="tg_bin_count failed with code -1"):
         _lib.check(lib.tg_bin_count(None, 0, None, -1, 64, 64, 16, 16, None, None), "tg_bin_count", bits)
 

@@ -12,7 +12,7 @@ Everything here calls the C ABI of libtrigrad_hip.so through trigrad_amd.
 import numpy as np
 import pytest
 
-from helpers import assert_close, to_device
+from helpers import assert_close, to_device, u64
 from test_gpu_stages import SCENES
 
 pytestmark = pytest.mark.gpu
@@ -249,6 +249,73 @@ def test_repeatable_and_stream_ordered(mode, cuda):
         for a, b in zip(first[2:], other[2:]):
             scale = float(a.abs().max())
             assert float((a - b).abs().max()) <= 1e-5 * scale + 1e-6
+
+
+@pytest.mark.parametrize("mode", ["A_default", "A_5_layers", "A_40_layers", "A_unlimited"])
+@pytest.mark.parametrize("name", ["soup_big_tris", "squares", "config0", "overlap_mesh_inf_w", "unit_square_negative_z"])
+def test_selection_early_stop_changes_nothing(name, mode, cuda, monkeypatch):
+    """With depth bounds of the lists the per-pixel selection may leave a list early; every output stays bit-identical."""
+    import torch
+    from trigrad_amd import _C
+    scene, tw, th = SCENES[name]()
+    m = MODES[mode]
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    ml = m["max_layers"] if m["max_layers"] > 0 else scene["indices"].shape[0] + 1
+    outs = []
+    for threshold in (1 << 30, 0):  # never / always
+        monkeypatch.setattr(_C, "EARLY_STOP_MIN_AVG_LIST", threshold)
+        outs.append(_C.render_forward(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, 1 / 256, True, True, ml))
+    for a, b in zip(outs[0][:7], outs[1][:7]):
+        assert torch.equal(a.view(torch.int32) if a.is_floating_point() else a, b.view(torch.int32) if b.is_floating_point() else b)
+    ra, rb = outs[0][8], outs[1][8]
+    assert torch.equal(ra[0], rb[0]) and torch.equal(ra[1].view(torch.int32), rb[1].view(torch.int32))
+    if ra[3] is not None:
+        layer = torch.arange(ra[3].shape[0], device=cuda)[:, None, None]
+        valid = layer < outs[0][6][None]
+        assert torch.equal(torch.where(valid, ra[3], 0), torch.where(valid, rb[3], 0))
+
+
+def test_list_bounds_values(cuda):
+    """tg_list_bounds: per tile and 256 entries, min over the rest of the list of (min z - 32 ulp max|z|); -inf where a
+    weight is not positive and finite."""
+    import torch
+    from trigrad_amd import _C, _lib, scenes as S
+    scene = S.random_soup(3000, 64, 48, seed=13, sigma_px=30.0, varying_w=True)
+    v = scene["vertices"].copy()
+    v[5, 3] = -1.0          # a negative weight
+    v[40, 3] = np.inf       # an infinite one
+    scene = dict(scene, vertices=v)
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    ids, offsets, keys, status = _C.per_tile_lists(d["vertices"], d["indices"], W, H, 16, 16)
+    T = _C.num_tiles(W, H, 16, 16)
+    K = ids.numel()
+    lib = _lib.load(32)
+    bounds = torch.full((int(lib.tg_list_bound_words(K, T)),), float("nan"), dtype=torch.float32, device=cuda)
+    far_start = torch.full((T,), -1, dtype=torch.int32, device=cuda)
+    low = torch.empty((scene["indices"].shape[0],), dtype=torch.float32, device=cuda)
+    _lib.check(lib.tg_list_bounds(_C._ptr(d["vertices"]), v.shape[0], _C._ptr(d["indices"]), scene["indices"].shape[0],
+                                  _C._ptr(keys), _C._ptr(ids), _C._ptr(offsets), T, _C._ptr(low), _C._ptr(bounds),
+                                  _C._ptr(far_start), _C._stream(ids)), "tg_list_bounds")
+    got, far_got = bounds.cpu().numpy(), far_start.cpu().numpy()
+    ids_h, off = ids.cpu().numpy(), offsets.cpu().numpy()
+    far = (u64(keys) & np.uint64(0xFFFFFFFF)) == np.uint64(np.array([1e30], np.float32).view(np.uint32)[0] ^ 0x80000000)
+    tri = v[scene["indices"][ids_h]]                       # (K,3,4)
+    z, w = tri[:, :, 2], tri[:, :, 3]
+    ok = ((w > 0) & np.isfinite(w) & np.isfinite(z)).all(axis=1)
+    lb = np.where(ok, z.min(axis=1) - np.float32(32) * np.finfo(np.float32).eps * np.abs(z).max(axis=1), -np.inf).astype(np.float32)
+    lb = np.where(far, np.float32(np.inf), lb)
+    assert far.any() and not far.all()
+    checked = 0
+    for t in range(T):
+        seg_far = far[off[t]:off[t + 1]]
+        assert far_got[t] == (int(np.argmax(seg_far)) if seg_far.any() else off[t + 1] - off[t])
+        for p in range(0, off[t + 1] - off[t], 256):
+            want = lb[off[t] + p:off[t + 1]].min()
+            assert got[off[t] // 256 + t + p // 256] == want
+            checked += 1
+    assert checked > T and (lb == -np.inf).any() and max(off[1:] - off[:-1]) > 256
 
 
 def test_record_timing_and_empty_scene(cuda):

@@ -91,6 +91,9 @@ SAVE_BLEND_ORDER = True
 # Without per_pixel_sort the forward pass saves which list entries cover which pixel (one bit per pair it
 # looked at) and the backward pass reads that back instead of repeating the inside tests.
 SAVE_HIT_MASKS = True
+# With per_pixel_sort and tile lists of at least this many entries on average, depth bounds of the lists are
+# computed (one more pass over the keys) so that the selection can stop before the end of a list.
+EARLY_STOP_MIN_AVG_LIST = 512
 
 
 def scan_exclusive(counts, out=None, heads=None):
@@ -314,6 +317,15 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             bary_transforms = cartesian_to_bary(vertices, indices)
 
         timer.start("rasterization")
+        batch_bounds = far_start = None
+        if per_pixel_sort and K >= EARLY_STOP_MIN_AVG_LIST * T:
+            # long lists: depth bounds let the selection leave a list before its end
+            batch_bounds = torch.empty((int(lib.tg_list_bound_words(K, T)),), dtype=real, device=dev)
+            far_start = torch.empty((T,), dtype=torch.int32, device=dev)
+            triangle_low = torch.empty((indices.shape[0],), dtype=real, device=dev)
+            _lib.check(lib.tg_list_bounds(_ptr(vertices), vertices.shape[0], _ptr(indices), indices.shape[0], _ptr(keys),
+                                          _ptr(sorted_ids), _ptr(offsets), T, _ptr(triangle_low), _ptr(batch_bounds),
+                                          _ptr(far_start), _stream(vertices)), "tg_list_bounds", bits)
         hit_masks = None
         if not per_pixel_sort and SAVE_HIT_MASKS:
             words = int(lib.tg_hit_mask_words(K, width, height, tile_width, tile_height))
@@ -322,7 +334,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
             width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
             _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
-            _ptr(hit_masks), _stream(vertices)), "tg_render_forward", bits)
+            _ptr(hit_masks), _ptr(batch_bounds), _ptr(far_start), _stream(vertices)), "tg_render_forward", bits)
         timings = timer.stop()
     return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
             (last, last_depth, sort_status, fragments, hit_masks))

@@ -39,8 +39,10 @@ SIGNATURES = {
     "tg_sort_pairs_u64_u32": (_i, [_p, _p, _p, _p, _i64, _i, _p, _sz, _p, C.POINTER(_i), _p]),
     "tg_tile_ranges": (_i, [_p, _i64, _i, _p, _p]),
     "tg_bary": (_i, [_p, _i32, _p, _i32, _p, _p]),
+    "tg_list_bound_words": (_sz, [_i64, _i]),
+    "tg_list_bounds": (_i, [_p, _i32, _p, _i32, _p, _p, _p, _i, _p, _p, _p, _p]),
     "tg_hit_mask_words": (_sz, [_i64, _i, _i, _i, _i]),
-    "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "tg_render_backward": (_i, [_p] * 17 + [_i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _i, _i, _i, _p]),
     "tg_barycentric": (None, [_p] * 5),
     "tg_barycentric_backward": (None, [_p] * 6),

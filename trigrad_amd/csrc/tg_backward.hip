@@ -821,7 +821,7 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
         set_error("tg_render_backward: vertices, image and grad_image must be 16-byte aligned");
         return TG_E_ARG;
     }
-    RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+    RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary, nullptr, nullptr,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
     BackwardArgs g{(const real4 *)grad_image, grad_depthmap, (const real4 *)image, depthmap, final_weights, ends, last,
                    last_depth, fragments, per_pixel_sort ? nullptr : hit_masks, grad_vertices, grad_colors, grad_opacities,

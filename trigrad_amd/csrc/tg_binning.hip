@@ -10,7 +10,7 @@
 //           coalesced
 //   ranges  reads 8 B per sorted key, writes 4 B per tile
 //   bary    reads 60 B, writes 36 B per triangle
-#include "tg_common.hpp"
+#include "tg_raster.hpp"
 
 namespace tg {
 
@@ -203,6 +203,101 @@ __global__ __launch_bounds__(kBinThreads) void tile_ranges_kernel(const uint64_t
     for (int t = prev + 1; t <= cur && t <= n_tiles; t++) offsets[t] = (int32_t)i;
 }
 
+// Lower bounds of the per-pixel depths (render.cu:404: interpolate3 of the vertex z with the vertex w
+// as weights) of the rest of every tile list, per batch of kBatch entries.  With positive finite
+// weights the interpolated depth is a convex combination of the three vertex depths, so it cannot lie
+// below their minimum by more than the rounding of the few operations involved; 32 ulps of the largest
+// |z| are subtracted for that.  An entry with a weight that is not positive and finite bounds nothing
+// (-inf).  Entries whose sort key is 1e30 (empty clipped polygon, render.cu:259) sit at the end of the
+// list whatever their depth: the bounds leave them out, far_start[tile] is the position of the first
+// one (the list length if there is none), and the reader looks at everything from there on.  The
+// double build's sorted keys no longer hold the depth, so nothing is left out there.
+// A first kernel writes every triangle's own bound; then one workgroup per tile: its waves take the
+// batches in turn and write each batch's own minimum, and the first wave turns those into minima over
+// the rest of the list, walking from the far end.
+constexpr int kBoundThreads = 256;
+
+__global__ __launch_bounds__(kBinThreads) void triangle_low_kernel(const real4 *__restrict__ vertices, int n_vertices,
+                                                                   const int32_t *__restrict__ indices, int n_triangles,
+                                                                   real *__restrict__ triangle_low) {
+    const int t = blockIdx.x * kBinThreads + threadIdx.x;
+    if (t >= n_triangles) return;
+    const real inf = std::numeric_limits<real>::infinity();
+    const int id[3] = {indices[3 * (int64_t)t], indices[3 * (int64_t)t + 1], indices[3 * (int64_t)t + 2]};
+    real zmin = inf, zabs = 0.0f;
+    bool ok = true;
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        ok = ok && (unsigned)id[k] < (unsigned)n_vertices;
+        const real4 v = ok ? vertices[id[k]] : make_real4(0.f, 0.f, 0.f, 0.f);
+        ok = ok && v.w > 0.0f && v.w < inf && abs_real(v.z) < inf;  // false for NaN as well
+        zmin = (v.z < zmin) ? v.z : zmin;
+        zabs = (abs_real(v.z) > zabs) ? abs_real(v.z) : zabs;
+    }
+    triangle_low[t] = ok ? zmin - 32.0f * std::numeric_limits<real>::epsilon() * zabs : -inf;
+}
+
+__global__ __launch_bounds__(kBoundThreads) void list_bounds_kernel(const real *__restrict__ triangle_low, int n_triangles,
+                                                                    const uint64_t *__restrict__ sorted_keys,
+                                                                    const int32_t *__restrict__ sorted_ids,
+                                                                    const int32_t *__restrict__ offsets,
+                                                                    real *__restrict__ bounds, int32_t *__restrict__ far_start) {
+    __shared__ int s_far;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int tile = blockIdx.x;
+    const int start = offsets[tile], n = offsets[tile + 1] - start;
+    const int n_batches = (n + kBatch - 1) / kBatch;
+    const real inf = std::numeric_limits<real>::infinity();
+    if (threadIdx.x == 0) s_far = n;
+    __syncthreads();
+    for (int b = wave; b < n_batches; b += kBoundThreads / kWave) {
+        real low = inf;
+        bool any_far = false;
+        int first_far = n;
+#pragma unroll
+        for (int c = kBatch / kWave - 1; c >= 0; c--) {
+            const int p = b * kBatch + c * kWave + lane;
+            real lb = inf;
+            bool far = false;
+            if (p < n) {
+#ifndef TG_DOUBLE_PRECISION
+                far = (uint32_t)sorted_keys[start + p] == orderable_bits(kFarKey);
+#endif
+                const int t = sorted_ids[start + p];
+                lb = far ? inf : ((unsigned)t < (unsigned)n_triangles ? triangle_low[t] : -inf);
+            }
+            const uint64_t far_lanes = __builtin_amdgcn_ballot_w64(far);
+            if (far_lanes) {
+                any_far = true;
+                first_far = b * kBatch + c * kWave + __builtin_ctzll(far_lanes);
+            }
+            low = (lb < low) ? lb : low;
+        }
+        low = wave_min(low);
+        if (lane == 0) {
+            bounds[batch_bound_index(start, tile, b * kBatch)] = low;
+            if (any_far) atomicMin(&s_far, first_far);
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+    if (wave != 0) return;
+    real rest = inf;  // bound of everything behind the batches in hand
+    for (int hi = n_batches; hi > 0; hi -= kWave) {
+        const int b = hi - 1 - lane;  // lane 0 holds the farthest batch
+        real v = (b >= 0) ? bounds[batch_bound_index(start, tile, b * kBatch)] : inf;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const real o = __shfl_up(v, d);
+            if (lane >= d) v = (o < v) ? o : v;
+        }
+        v = (rest < v) ? rest : v;
+        if (b >= 0) bounds[batch_bound_index(start, tile, b * kBatch)] = v;
+        rest = __shfl(v, kWave - 1);
+    }
+    if (lane == 0) far_start[tile] = s_far;
+}
+
 // render.cu:310-337 cartesian_to_bary_kernel.
 __global__ __launch_bounds__(kBinThreads) void bary_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                            const int32_t *__restrict__ indices, int n_triangles,
@@ -284,4 +379,27 @@ extern "C" int tg_bary(const real *vertices, int32_t n_vertices, const int32_t *
     TG_LAUNCH(bary_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
                        (const real4 *)vertices, n_vertices, indices, n_triangles, out);
     return check_launch("bary_kernel");
+}
+
+extern "C" size_t tg_list_bound_words(int64_t n_keys, int n_tiles) {
+    if (n_keys < 0 || n_tiles <= 0) return 0;
+    return (size_t)(n_keys / kBatch + n_tiles + 1);
+}
+
+extern "C" int tg_list_bounds(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles,
+                              const uint64_t *sorted_keys, const int32_t *sorted_ids, const int32_t *offsets, int n_tiles,
+                              real *triangle_low, real *bounds, int32_t *far_start, void *stream) {
+    if (n_tiles <= 0 || n_vertices < 0 || n_triangles < 0 || !offsets || !bounds || !far_start || ((uintptr_t)vertices & 15) ||
+        (n_triangles > 0 && (!vertices || !indices || !triangle_low))) {
+        set_error("tg_list_bounds: null pointer, non-positive tile count or misaligned vertices");
+        return TG_E_ARG;
+    }
+    if (n_triangles > 0) {
+        TG_LAUNCH(triangle_low_kernel, dim3(ceil_div(n_triangles, kBinThreads)), dim3(kBinThreads), 0, (hipStream_t)stream,
+                  (const real4 *)vertices, n_vertices, indices, n_triangles, triangle_low);
+        if (int e = check_launch("triangle_low_kernel")) return e;
+    }
+    TG_LAUNCH(list_bounds_kernel, dim3(n_tiles), dim3(kBoundThreads), 0, (hipStream_t)stream, triangle_low, n_triangles,
+              sorted_keys, sorted_ids, offsets, bounds, far_start);
+    return check_launch("list_bounds_kernel");
 }

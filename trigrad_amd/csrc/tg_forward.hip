@@ -141,6 +141,20 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         int found = 0;
         for (int batch = start; batch < end; batch += kBatch) {
             const int nb = min(kBatch, end - batch);
+            if (a.batch_bounds) {
+                // a lane needs nothing from here on when its list is full and its worst candidate is nearer than
+                // every fragment the rest of the tile's list can produce (a full list rejects depths >= its worst)
+                const real rest = a.batch_bounds[batch_bound_index(start, tile, batch - start)];
+                const bool settled = !want || (found == cap && tk.d(cap - 1) <= rest);
+                if (__syncthreads_and(settled)) {
+                    // on to the batch that holds the first entry the bounds do not cover
+                    const int resume = start + a.far_start[tile] / kBatch * kBatch;
+                    if (resume > batch) {
+                        batch = resume - kBatch;
+                        continue;
+                    }
+                }
+            }
             __syncthreads();
             for (int e = tid; e < nb; e += blockDim.x) {
                 gather_depth(a, batch + e, s_rec[e]);
@@ -300,7 +314,8 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
                                  const int32_t *sorted_ids, const int32_t *offsets, const real *bary, int width, int height,
                                  int tile_w, int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers,
                                  real *image, real *depthmap, real *final_weights, int32_t *ends, int32_t *last,
-                                 real *last_depth, int32_t *fragments, uint64_t *hit_masks, void *stream) {
+                                 real *last_depth, int32_t *fragments, uint64_t *hit_masks, const real *batch_bounds,
+                                 const int32_t *far_start, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
         set_error("tg_render_forward: null pointer");
@@ -311,7 +326,12 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         return TG_E_ARG;
     }
     RasterArgs a{(const real4 *)vertices, indices, colors, opacities, sorted_ids, offsets, bary,
+                 per_pixel_sort ? batch_bounds : nullptr, (per_pixel_sort && batch_bounds) ? far_start : nullptr,
                  width, height, tile_w, tile_h, early_stopping_threshold, max_layers};
+    if (batch_bounds && !far_start) {
+        set_error("tg_render_forward: batch_bounds come with far_start");
+        return TG_E_ARG;
+    }
     if (fragments && (!per_pixel_sort || max_layers > TG_MAX_SAVED_LAYERS)) {
         set_error("tg_render_forward: fragments are saved only with per_pixel_sort and max_layers <= %d", TG_MAX_SAVED_LAYERS);
         return TG_E_ARG;

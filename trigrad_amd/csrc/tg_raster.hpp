@@ -27,6 +27,8 @@ struct RasterArgs {
     const int32_t *sorted_ids;
     const int32_t *offsets;
     const real *bary;
+    const real *batch_bounds;  // per tile and batch of kBatch entries: lower bound of the pixel depths from there on; may be null
+    const int32_t *far_start;  // per tile: first list position whose entries the bounds do not cover (with batch_bounds)
     int W, H, tw, th;
     real thr;
     int max_layers;
@@ -117,6 +119,17 @@ __device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRe
 // n_keys / 64 + n_tiles + 1 chunks hold every list.
 __device__ __forceinline__ int64_t hit_mask_chunk(int start, int tile, int relative_position) {
     return (int64_t)(start >> 6) + tile + (relative_position >> 6);
+}
+
+// Batch bounds: word batch_bound_index(start, tile, p) holds, for the tile whose
+// list starts at `start`, a lower bound of the per-pixel depth of every entry at
+// relative position >= p (p a multiple of kBatch) and < far_start[tile].  From
+// far_start on the list holds the entries whose clipped polygon was empty (sort
+// key 1e30): they lie at the end of the list whatever their depth, almost never
+// cover a pixel, and are always looked at.  Tiles never share a word;
+// n_keys / kBatch + n_tiles + 1 words hold every list.
+__device__ __forceinline__ int64_t batch_bound_index(int start, int tile, int relative_position) {
+    return (int64_t)(start / kBatch) + tile + relative_position / kBatch;
 }
 
 // Front-to-back compositing state of one pixel (render.cu:564-574).
