@@ -44,12 +44,13 @@ struct alignas(16) BackRecord {
     real m[9];
     real w[3];
     real iw[3];
+    real iw2[3];  // 1 / (w * w)
     real op[3];
     real col[9];
-    real xy[6];  // ax, ay, bx, by, cx, cy
+    real xy[6];   // ax, ay, bx, by, cx, cy
     int id[3];
 };
-constexpr int kBackReals = 33;  // scalars in front of the ids
+constexpr int kBackReals = 36;  // scalars in front of the ids
 static_assert(offsetof(BackRecord, id) == kBackReals * sizeof(real), "BackRecord layout");
 
 __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackRecord &r) {
@@ -60,6 +61,7 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
     const real4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
     r.iw[0] = 1.0f / va.w; r.iw[1] = 1.0f / vb.w; r.iw[2] = 1.0f / vc.w;
+    r.iw2[0] = 1.0f / (va.w * va.w); r.iw2[1] = 1.0f / (vb.w * vb.w); r.iw2[2] = 1.0f / (vc.w * vc.w);
     r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
 #pragma unroll
     for (int k = 0; k < 3; k++) {
@@ -70,6 +72,16 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
     r.xy[0] = va.x; r.xy[1] = va.y; r.xy[2] = vb.x; r.xy[3] = vb.y; r.xy[4] = vc.x; r.xy[5] = vc.y;
     r.id[0] = t.ia; r.id[1] = t.ib; r.id[2] = t.ic;
 }
+
+// 1 / x to within one unit in the last place: the hardware estimate and one Newton step where
+// the estimate is an ordinary number (zero, infinity and NaN pass through as they are).  Used
+// where the reference divides in its backward pass and the quotient is no carried state.
+__device__ __forceinline__ float reciprocal(float x) {
+    const float r = __builtin_amdgcn_rcpf(x);
+    const float refined = __builtin_fmaf(__builtin_fmaf(-x, r, 1.0f), r, r);
+    return __builtin_amdgcn_classf(r, 0x198) ? refined : r;  // +-normal, +-denormal
+}
+__device__ __forceinline__ double reciprocal(double x) { return 1.0 / x; }
 
 // Reverse-traversal state of one pixel (render.cu:647-653).
 struct BackState {
@@ -85,18 +97,16 @@ __device__ __forceinline__ void interp_backward_scalar(real g, const real b[3], 
                                                        real gb[3], real gv[3], real gw[3]) {
     const real nom = (b[0] * w[0] * v[0] + b[1] * w[1] * v[1]) + b[2] * w[2] * v[2];
     const real denom = (b[0] * w[0] + b[1] * w[1]) + b[2] * w[2];
-    if (denom * denom < kEffZero) {
-#pragma unroll
-        for (int k = 0; k < 3; k++) gb[k] = gv[k] = gw[k] = 0.0f;
-        return;
-    }
-    const real inv2 = 1.0f / (denom * denom);
-    const real inv = 1.0f / denom;  // shared by the three value gradients (the reference divides three times)
+    // all zero where the reference returns early (util.h:303); written as selections, because a branch
+    // around the assignments of three arrays makes the compiler keep them in scratch memory
+    const bool dead = denom * denom < kEffZero;
+    const real inv = reciprocal(denom);  // the reference divides nine times, by denom and by its square
+    const real inv2 = inv * inv;
 #pragma unroll
     for (int k = 0; k < 3; k++) {
-        gb[k] = g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
-        gv[k] = g * b[k] * w[k] * inv;
-        gw[k] = g * (b[k] * v[k] * denom - nom * b[k]) * inv2;
+        gb[k] = dead ? 0.0f : g * ((v[k] * w[k] * denom - nom * w[k]) * inv2);
+        gv[k] = dead ? 0.0f : g * b[k] * w[k] * inv;
+        gw[k] = dead ? 0.0f : g * (b[k] * v[k] * denom - nom * b[k]) * inv2;
     }
 }
 
@@ -114,22 +124,32 @@ struct FragSeed {
     real dd_dz;   // derivative w.r.t. the interpolated view depth (:517)
 };
 
-__device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, real b0, real b1, real b2) {
+// The fragment itself: interpolated opacity, colour and view depth (no state involved).
+struct FragValue {
+    real o, color[3], z;
+};
+
+__device__ __forceinline__ FragValue fragment_value(const BackRecord &r, real b0, real b1, real b2) {
     const real w[3] = {r.w[0], r.w[1], r.w[2]};
+    FragValue v;
     // The opacity is recomputed exactly as the forward pass computed it: 1 - o can be small, and the
     // transmittance is reconstructed by dividing by it.  The three colour quotients over the same
     // denominator (util.h:245-250) share its reciprocal.
-    real o = interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]);
-    o = clampf(o, 0.0f, kMaxOpacity);
-    const real inv_denom = 1.0f / (b0 * w[0] + b1 * w[1] + b2 * w[2]);
-    real color[3];
+    v.o = clampf(interp_w(b0, b1, b2, r.op[0], r.op[1], r.op[2], w[0], w[1], w[2]), 0.0f, kMaxOpacity);
+    const real inv_denom = reciprocal(b0 * w[0] + b1 * w[1] + b2 * w[2]);
 #pragma unroll
     for (int k = 0; k < 3; k++)
-        color[k] = (b0 * r.col[k] * w[0] + b1 * r.col[3 + k] * w[1] + b2 * r.col[6 + k] * w[2]) * inv_denom;
-    const real z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+        v.color[k] = (b0 * r.col[k] * w[0] + b1 * r.col[3 + k] * w[1] + b2 * r.col[6 + k] * w[2]) * inv_denom;
+    v.z = interp_1(b0, b1, b2, r.iw[0], r.iw[1], r.iw[2]);
+    return v;
+}
 
+// The step from one fragment of a pixel to the next one in reverse blend order (render.cu:487-517).
+__device__ __forceinline__ FragSeed fragment_chain_step(BackState &st, const FragValue &v) {
+    const real o = v.o, z = v.z;
+    const real color[3] = {v.color[0], v.color[1], v.color[2]};
     const real om = 1.0f - o;
-    const real inv_om = 1.0f / om;  // the reference divides six derivative terms by om; they share this reciprocal
+    const real inv_om = reciprocal(om);  // the reference divides six derivative terms by om
     const real g[3] = {st.g0, st.g1, st.g2};
     real s[3] = {st.s0, st.s1, st.s2};
     real t3[3];
@@ -155,6 +175,10 @@ __device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const Bac
     return f;
 }
 
+__device__ __forceinline__ FragSeed fragment_state_step(BackState &st, const BackRecord &r, real b0, real b1, real b2) {
+    return fragment_chain_step(st, fragment_value(r, b0, b1, b2));
+}
+
 // The order-free part: the 21 gradient terms of one fragment.
 __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackRecord &r, real b0, real b1, real b2, real px,
                                                real py, real out[kTerms]) {
@@ -166,28 +190,27 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
 
     // vector interpolate3_backward for the colour (util.h:319-355)
     const real *gc = f.gc;
-    real gb_c[3] = {0.f, 0.f, 0.f}, gw_c[3] = {0.f, 0.f, 0.f}, scale[3] = {0.f, 0.f, 0.f};
+    real gb_c[3], gw_c[3], scale[3];
     {
         real nom[3];
 #pragma unroll
         for (int k = 0; k < 3; k++) nom[k] = (b[0] * w[0] * r.col[k] + b[1] * w[1] * r.col[3 + k]) + b[2] * w[2] * r.col[6 + k];
         const real denom = b[0] * w[0] + b[1] * w[1] + b[2] * w[2];
-        if (!(denom * denom < kEffZero)) {
-            const real inv2 = 1.0f / (denom * denom);
-            const real inv = 1.0f / denom;
+        const bool dead = denom * denom < kEffZero;  // util.h:326: all zero (selections, not a branch: see above)
+        const real inv = reciprocal(denom);
+        const real inv2 = inv * inv;
 #pragma unroll
-            for (int v = 0; v < 3; v++) {
-                real dfb[3], dfw[3];
+        for (int v = 0; v < 3; v++) {
+            real dfb[3], dfw[3];
 #pragma unroll
-                for (int k = 0; k < 3; k++) {
-                    const real a = r.col[3 * v + k];
-                    dfb[k] = w[v] * (a * denom - nom[k]) * inv2;
-                    dfw[k] = (b[v] * a * denom - nom[k] * b[v]) * inv2;
-                }
-                gb_c[v] = (gc[0] * dfb[0] + gc[1] * dfb[1]) + gc[2] * dfb[2];
-                gw_c[v] = (gc[0] * dfw[0] + gc[1] * dfw[1]) + gc[2] * dfw[2];
-                scale[v] = b[v] * w[v] * inv;
+            for (int k = 0; k < 3; k++) {
+                const real a = r.col[3 * v + k];
+                dfb[k] = w[v] * (a * denom - nom[k]) * inv2;
+                dfw[k] = (b[v] * a * denom - nom[k] * b[v]) * inv2;
             }
+            gb_c[v] = dead ? 0.0f : (gc[0] * dfb[0] + gc[1] * dfb[1]) + gc[2] * dfb[2];
+            gw_c[v] = dead ? 0.0f : (gc[0] * dfw[0] + gc[1] * dfw[1]) + gc[2] * dfw[2];
+            scale[v] = dead ? 0.0f : b[v] * w[v] * inv;
         }
     }
 
@@ -200,19 +223,23 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
 
     // util.h:405-455 barycentric_backward (vertex part)
     const real ax = r.xy[0], ay = r.xy[1], bx = r.xy[2], by = r.xy[3], cx = r.xy[4], cy = r.xy[5];
-    real dxy[3][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    real dxy[3][2];
     {
         // The reference divides each of the 21 numerators below by T or d (util.h:405-455).  Here the two
-        // reciprocals are formed once (correctly rounded) and multiplied in: every quotient is within one ulp
-        // of the reference's instead of half an ulp, and 19 of the fragment's 50 divisions go away.
+        // reciprocals are formed once and multiplied in: every quotient is within two units in the last
+        // place of the reference's, and 19 of the fragment's 50 divisions go away.  The numerators keep the
+        // reference's form: its differences of screen coordinates cancel, and for a sliver that rounding
+        // is larger than the tolerance of the comparison, so the shorter closed form
+        // (-l_v * row k of the matrix) does not reproduce the reference's numbers.
         const real T = (bx - ax) * (cy - ay) - (by - ay) * (cx - ax);
-        const real inv_T = 1.0f / T;
+        const real inv_T = reciprocal(T);
         const real l0 = ((bx - px) * (cy - py) - (by - py) * (cx - px)) * inv_T;
         const real l1 = ((cx - px) * (ay - py) - (cy - py) * (ax - px)) * inv_T;
         const real l2 = ((ax - px) * (by - py) - (ay - py) * (bx - px)) * inv_T;
         const real d = ax * (by - cy) + bx * (-ay + cy) + cx * (ay - by);
-        if (!(abs_real(d) < kEffZero)) {
-            const real inv_d = 1.0f / d;
+        const bool flat = abs_real(d) < kEffZero;  // util.h:421: zero (selection, not a branch: see above)
+        {
+            const real inv_d = reciprocal(d);
             real J[3][2][3];
             J[0][0][0] = l0 * (-by + cy) * inv_d;
             J[0][0][1] = (-cy - l1 * (by - cy) + py) * inv_d;
@@ -235,12 +262,12 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
 #pragma unroll
             for (int v = 0; v < 3; v++)
 #pragma unroll
-                for (int c = 0; c < 2; c++) dxy[v][c] = gbary[0] * J[v][c][0] + gbary[1] * J[v][c][1] + gbary[2] * J[v][c][2];
+                for (int c = 0; c < 2; c++) dxy[v][c] = flat ? 0.0f : gbary[0] * J[v][c][0] + gbary[1] * J[v][c][1] + gbary[2] * J[v][c][2];
         }
     }
 #pragma unroll
     for (int v = 0; v < 3; v++) {
-        const real dd_dw = -gv_z[v] / (w[v] * w[v]);   // :523-525
+        const real dd_dw = -gv_z[v] * r.iw2[v];        // :523-525
         const real dw = gw_o[v] + gw_c[v] + gw_z[v];   // :530
         out[7 * v + 0] = dxy[v][0];
         out[7 * v + 1] = dxy[v][1];
@@ -482,6 +509,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
         wave_lds_sync();
 
         for (uint32_t round0 = 0; round0 < n_hits; round0 += kWaveSlots) {
+            const int n_slots = (int)min((uint32_t)kWaveSlots, n_hits - round0);
             // 3. ordered part, lane by lane over its own hits
             while (true) {
                 int e = -1;
@@ -490,10 +518,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 else if (m[0]) e = top_bit(m[0]);
                 if (e >= 0) {
                     slot = bases[e] + lanes_below_mask(ballots[e]) - round0;
-                    if (slot >= (uint32_t)kWaveSlots) e = -1;  // this hit, and all my later ones, belong to a later round
+                    if (slot >= (uint32_t)kWaveSlots) e = -1;
                 }
                 const bool active = e >= 0;
-                if (__builtin_amdgcn_ballot_w64(active) == 0) break;  // wave-uniform
+                if (__builtin_amdgcn_ballot_w64(active) == 0) break;
                 if (active) {
                     if (e >= 64) m[1] &= ~(1ull << (e - 64)); else m[0] &= ~(1ull << e);
                     const BackRecord &r = s_rec[e];
@@ -511,7 +539,6 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
             wave_lds_sync();
 
             // 4. order-free part
-            const int n_slots = (int)min((uint32_t)kWaveSlots, n_hits - round0);
             for (int s0 = 0; s0 < n_slots; s0 += kWave) {
                 const int n_here = min(kWave, n_slots - s0);
                 int tag = -1;
@@ -689,7 +716,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 // entries beyond the staged window are gathered from and added to memory
 // directly.
 constexpr int kSavedWindow = 256;
-constexpr int kSavedStride = kBackReals + 4;  // 33 scalars, 3 vertex ids; odd
+constexpr int kSavedStride = kBackReals + 3;  // 36 scalars, 3 vertex ids; odd
 
 template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
