@@ -28,6 +28,8 @@ def _scenes():
         "unit_square_negative_z": lambda: (S.unit_square(), 16, 16),
         "overlap_mesh_inf_w": lambda: (S.overlap_mesh(), 16, 16),
         "grid_mesh": lambda: (S.grid_mesh(40, 40, -0.9, 0.9, -0.9, 0.9, width=96, height=96), 16, 16),
+        # every border tile, the first one included, has an empty list and nothing to walk back
+        "center_island": lambda: (S.grid_mesh(12, 12, -0.3, 0.3, -0.3, 0.3, width=128, height=96), 16, 16),
     }
     return out
 

@@ -292,14 +292,19 @@ __device__ __forceinline__ void fragment_backward(BackState &st, const BackRecor
 enum GradLayout { kGradDense = 0, kGradBlock8 = 1, kGradStrided = 2 };
 
 template <int kLayout>
+__device__ __forceinline__ int term_stride(const BackwardArgs &g, int c) {
+    if (c < 3) return kLayout == kGradDense ? 4 : kLayout == kGradBlock8 ? 8 : g.vertex_stride;
+    if (c < 6) return kLayout == kGradDense ? 3 : kLayout == kGradBlock8 ? 8 : g.color_stride;
+    return kLayout == kGradDense ? 1 : kLayout == kGradBlock8 ? 8 : g.opacity_stride;
+}
+
+template <int kLayout>
 __device__ __forceinline__ real *term_address(const BackwardArgs &g, int vertex_id, int c) {
-    const int sv = kLayout == kGradDense ? 4 : kLayout == kGradBlock8 ? 8 : g.vertex_stride;
-    const int sc = kLayout == kGradDense ? 3 : kLayout == kGradBlock8 ? 8 : g.color_stride;
-    const int so = kLayout == kGradDense ? 1 : kLayout == kGradBlock8 ? 8 : g.opacity_stride;
-    if (c < 2) return g.grad_vertices + sv * (int64_t)vertex_id + c;
-    if (c == 2) return g.grad_vertices + sv * (int64_t)vertex_id + 3;
-    if (c < 6) return g.grad_colors + sc * (int64_t)vertex_id + (c - 3);
-    return g.grad_opacities + so * (int64_t)vertex_id;
+    const int64_t at = term_stride<kLayout>(g, c) * (int64_t)vertex_id;
+    if (c < 2) return g.grad_vertices + at + c;
+    if (c == 2) return g.grad_vertices + at + 3;
+    if (c < 6) return g.grad_colors + at + (c - 3);
+    return g.grad_opacities + at;
 }
 
 __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, const PixelCoord &p) {
@@ -317,37 +322,6 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
     return st;
 }
 
-// Adds up, in slot order, the runs of equal tag among slots [c0, c1) of one row
-// of a term matrix and hands every non-zero run sum to flush(tag, sum).  Tags and
-// terms are read eight slots ahead, so the LDS latency is paid once per eight
-// slots instead of once per slot.
-template <typename TagAt, typename Flush>
-__device__ __forceinline__ void sum_runs(const real *row, int c0, int c1, TagAt tag_at, Flush flush) {
-    constexpr int kAhead = 8;
-    int cur = tag_at(c0);
-    real sum = 0.0f;
-    for (int c = c0; c < c1; c += kAhead) {
-        int t[kAhead];
-        real v[kAhead];
-#pragma unroll
-        for (int k = 0; k < kAhead; k++) {
-            const int i = min(c + k, c1 - 1);
-            t[k] = tag_at(i);
-            v[k] = row[i];
-        }
-#pragma unroll
-        for (int k = 0; k < kAhead; k++) {
-            if (c + k >= c1) break;
-            if (t[k] != cur) {
-                if (sum != 0.0f) flush(cur, sum);
-                sum = 0.0f;
-                cur = t[k];
-            }
-            sum += v[k];
-        }
-    }
-    if (sum != 0.0f) flush(cur, sum);
-}
 
 constexpr int kBackBatch = 128;   // list entries staged per batch
 constexpr int kWaveSlots = 256;   // hit slots per wave and round
@@ -355,10 +329,26 @@ constexpr int kSeedWords = 6;     // d_do, gc[3], dd_dz, (entry | source lane <<
 constexpr int kTermStride = 65;   // row stride of the per-wave term matrix (odd: conflict-free columns)
 constexpr int kMaxWaves = kTileThreads / kWave;
 
-__device__ __forceinline__ int top_bit(uint64_t m) { return 63 - __builtin_clzll(m); }
+// The run sums' view of a lane: lane = 21 * group + q adds up gradient term q over the group's third
+// of the slots.  What depends on q only is worked out once per kernel.
+struct TermLane {
+    int group;   // 0..2; 3 for the one lane left over
+    int q;
+    int vertex;  // q / 7: which of the entry's three vertices the term belongs to
+    int stride;  // scalars per vertex in the term's array
+    real *base;  // the term's element of vertex 0
+};
 
-__device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
-    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+template <int kLayout>
+__device__ __forceinline__ TermLane term_lane(const BackwardArgs &g, int lane) {
+    TermLane t;
+    t.group = lane / kTerms;
+    t.q = lane - t.group * kTerms;
+    t.vertex = t.q / 7;
+    const int c = t.q - 7 * t.vertex;
+    t.stride = term_stride<kLayout>(g, c);
+    t.base = term_address<kLayout>(g, 0, c);
+    return t;
 }
 
 // Orders the LDS traffic of one wave: what lanes wrote before is visible to the
@@ -368,6 +358,74 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Adds up the runs of equal list entry among the first n slots of a wave's term matrix (row q = term
+// q, rows kTermStride apart; slots of one entry are neighbours) and adds every non-zero run sum to the
+// gradient arrays.  Bit c of `heads` is set where slot c starts a run.  First every lane (group, q)
+// turns its third of row q into running sums that start over at each head: no branch and no look at
+// the entries.  The last slot of a run, and of a third, then holds a sum to deliver; those slots are
+// taken three at a time, one per group.  entry_at(c): list entry of slot c; vertex_of(entry, v):
+// vertex id v of that entry.
+template <typename EntryAt, typename VertexOf>
+__device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads, const TermLane &t, EntryAt entry_at,
+                                             VertexOf vertex_of) {
+    constexpr int kAhead = 8;  // terms read ahead, so that the LDS latency is paid once per eight slots
+    const int per = (n + 2) / 3;
+    const int c0 = min(t.group * per, n), c1 = min(c0 + per, n);
+    real *row = terms + t.q * kTermStride;
+    if (t.group < 3) {
+        const uint32_t mine = (uint32_t)(heads >> c0);  // per <= 22 slots
+        real sum = 0.0f;
+        for (int i = 0; c0 + i < c1; i += kAhead) {
+            real v[kAhead];
+#pragma unroll
+            for (int k = 0; k < kAhead; k++) v[k] = row[min(c0 + i + k, c1 - 1)];
+#pragma unroll
+            for (int k = 0; k < kAhead; k++) {
+                if (c0 + i + k >= c1) break;
+                sum = ((mine >> (i + k)) & 1) ? v[k] : sum + v[k];
+                row[c0 + i + k] = sum;
+            }
+        }
+    }
+    wave_lds_sync();
+    uint64_t tails = (heads >> 1) | (1ull << (n - 1));
+    if (per < n) tails |= 1ull << (per - 1);
+    if (2 * per < n) tails |= 1ull << (2 * per - 1);
+    if (n < kWave) tails &= (1ull << n) - 1;
+    while (tails) {  // wave-uniform; six slots per turn, so that two chains of LDS reads are in flight per lane
+        int c[2] = {-1, -1};
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int k = 0; k < 3; k++)
+                if (tails) {
+                    const int bit = __builtin_ctzll(tails);
+                    tails &= tails - 1;
+                    if (t.group == k) c[u] = bit;
+                }
+        real sum[2] = {0.0f, 0.0f};
+        int entry[2] = {0, 0}, vertex[2] = {0, 0};
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            if (c[u] >= 0) {
+                sum[u] = row[c[u]];
+                entry[u] = entry_at(c[u]);
+            }
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            if (c[u] >= 0) vertex[u] = vertex_of(entry[u], t.vertex);
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            if (sum[u] != 0.0f) unsafeAtomicAdd(t.base + (int64_t)t.stride * vertex[u], sum[u]);
+    }
+}
+
+__device__ __forceinline__ int top_bit(uint64_t m) { return 63 - __builtin_clzll(m); }
+
+__device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
 // Tile-order backward.  LDS floating-point atomics cost about three cycles per lane on
@@ -407,56 +465,83 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile];
     const PixelCoord p = pixel_of_thread(a);
+    const TermLane tl = term_lane<kLayout>(g, lane);
     uint64_t *ballots = s_ballot[wave];
     uint32_t *bases = s_base[wave];
     real (*seeds)[kWaveSlots] = s_seed[wave];
     real *terms = s_term[wave];
 
-    // the pixel's loads are issued before the barriers below, which then cover their latency
+    // With the forward pass's masks comes the number of list entries this workgroup has to walk; else
+    // it is the largest `last` of its pixels.  The pixel's own loads are issued first either way: the
+    // barriers and the staging of the first batch cover their latency.
+    const bool saved_masks = g.hit_masks != nullptr;
+    const uint64_t *const masks = saved_masks ? g.hit_masks + hit_mask_head_words() : nullptr;
     const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
     BackState st;
     if (p.valid) st = load_back_state(g, p);
-    if (tid == 0) s_last = 0;
     s_px[tid] = p.px;
     s_py[tid] = p.py;
-    if (!g.hit_masks) publish_wave_rect(p, s_rects);  // only the repeated inside tests cull by wave rectangle
-    __syncthreads();
-    if (my_last > 0) atomicMax(&s_last, my_last);
-    __syncthreads();
-    const int tile_last = s_last;
+    int tile_last;
+    if (saved_masks) {
+        tile_last = (int)g.hit_masks[hit_mask_head_index()];
+    } else {
+        if (tid == 0) s_last = 0;
+        publish_wave_rect(p, s_rects);  // only the repeated inside tests cull by wave rectangle
+        __syncthreads();
+        if (my_last > 0) atomicMax(&s_last, my_last);
+        __syncthreads();
+        tile_last = s_last;
+    }
 
     // Batches are aligned to multiples of kBackBatch from the start of the list (the last one may be
     // short), so that a batch is two whole words of the saved hit masks.
-    const bool saved_masks = g.hit_masks != nullptr;
     const int64_t mask_slots = (int64_t)gridDim.z * blockDim.x, mask_slot = (int64_t)blockIdx.z * blockDim.x + tid;
-    for (int hi = (tile_last + kBackBatch - 1) / kBackBatch * kBackBatch; hi > 0; hi -= kBackBatch) {
+    // A workgroup with a thread per staged entry keeps the entry of the next batch in registers: its
+    // loads are issued when a batch starts and land in LDS when the next one does.
+    const bool ahead = (int)blockDim.x >= kBackBatch;
+    const int hi0 = (tile_last + kBackBatch - 1) / kBackBatch * kBackBatch;
+    BackRecord next;
+    if (ahead && hi0 > 0 && tid < tile_last - (hi0 - kBackBatch)) gather_back(a, start + hi0 - kBackBatch + tid, next);  // hi0 = 0: nothing to walk
+    for (int hi = hi0; hi > 0; hi -= kBackBatch) {
         const int lo = hi - kBackBatch;
         const int nb = min(hi, tile_last) - lo;
+        const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
+        // my saved masks of the batch: asked for here, used after the staging
+        uint64_t m[2] = {0, 0};
+        if (saved_masks) {
+            const int64_t chunk = hit_mask_chunk(start, tile, lo);
+#pragma unroll
+            for (int wd = 0; wd < 2; wd++)
+                if (64 * wd < mine) {
+                    m[wd] = masks[(chunk + wd) * mask_slots + mask_slot];
+                    if (mine < 64 * wd + 64) m[wd] &= (1ull << (mine - 64 * wd)) - 1;  // entries past my last one
+                }
+        }
         __syncthreads();  // every wave is done with the previous batch
-        for (int e = tid; e < nb; e += blockDim.x) {
-            gather_back(a, start + lo + e, s_rec[e]);
-            if (!saved_masks) s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+        if (ahead) {
+            if (tid < nb) {
+                s_rec[tid] = next;
+                if (!saved_masks) s_touch[tid] = (uint8_t)waves_touched(next.m, s_rects, n_waves);
+            }
+            if (lo > 0 && tid < kBackBatch) gather_back(a, start + lo - kBackBatch + tid, next);  // all batches but the first are full
+        } else {
+            for (int e = tid; e < nb; e += blockDim.x) {
+                gather_back(a, start + lo + e, s_rec[e]);
+                if (!saved_masks) s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+            }
         }
         __syncthreads();
 
         // 1. which entries cover which pixel: read back what the forward pass saved, or test again
         //    (then only the entries that can touch this wave's pixels)
-        const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
         if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
         ballots[lane] = 0;
         ballots[lane + kWave] = 0;
         wave_lds_sync();
-        uint64_t m[2] = {0, 0};
         if (saved_masks) {
-            const int64_t chunk = hit_mask_chunk(start, tile, lo);
 #pragma unroll
             for (int wd = 0; wd < 2; wd++) {
-                uint64_t bits = 0;
-                if (64 * wd < mine) {
-                    bits = g.hit_masks[(chunk + wd) * mask_slots + mask_slot];
-                    if (mine < 64 * wd + 64) bits &= (1ull << (mine - 64 * wd)) - 1;  // entries past my last one
-                }
-                m[wd] = bits;
+                const uint64_t bits = m[wd];
                 // per-entry ballots = the transpose, for the entries any lane holds
                 uint32_t any_lo = (uint32_t)bits, any_hi = (uint32_t)(bits >> 32);
 #pragma unroll
@@ -562,15 +647,11 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
 #pragma unroll
                     for (int q = 0; q < kTerms; q++) terms[q * kTermStride + lane] = term[q];
                 }
+                const int tag_before = __shfl_up(tag, 1, kWave);
+                const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_here && (lane == 0 || tag != tag_before));
                 wave_lds_sync();
-                // lanes (group, q): group 0..2 owns a third of the slots; runs of equal entry are contiguous
-                const int group = lane / kTerms, q = lane - group * kTerms;
-                const int per = (n_here + 2) / 3;
-                const int c0 = group * per, c1 = min(c0 + per, n_here);
-                if (group < 3 && c0 < c1)
-                    sum_runs(terms + q * kTermStride, c0, c1,
-                             [&](int c) { return int_of_real(seeds[5][s0 + c]) & 0xff; },
-                             [&](int entry, real sum) { unsafeAtomicAdd(term_address<kLayout>(g, s_rec[entry].id[q / 7], q % 7), sum); });
+                add_run_sums(terms, n_here, heads, tl, [&](int c) { return int_of_real(seeds[5][s0 + c]) & 0xff; },
+                             [&](int entry, int v) { return s_rec[entry].id[v]; });
                 wave_lds_sync();
             }
         }
@@ -742,6 +823,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     __syncthreads();
     real *terms = s_term[wave];
     int *tags = s_tag[wave];
+    const TermLane tl = term_lane<kLayout>(g, lane);
 
     BackState st;
     int n = 0;
@@ -805,14 +887,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
                 tags[slot] = rel[u];
             }
             wave_lds_sync();
-            // lanes (group, q): group 0..2 owns a third of the slots; runs of equal entry are contiguous
-            const int group = lane / kTerms, q = lane - group * kTerms;
-            const int per = (n_slots + 2) / 3;
-            const int c0 = group * per, c1 = min(c0 + per, n_slots);
-            if (group < 3 && c0 < c1)
-                sum_runs(terms + q * kTermStride, c0, c1, [&](int c) { return tags[c]; }, [&](int entry, real sum) {
-                    unsafeAtomicAdd(term_address<kLayout>(g, int_of_real(s_rows[entry * kSavedStride + kBackReals + q / 7]), q % 7), sum);
-                });
+            // a slot starts a run where its entry differs from the slot before
+            const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tags[lane] != tags[max(lane - 1, 0)]));
+            add_run_sums(terms, n_slots, heads, tl, [&](int c) { return tags[c]; },
+                         [&](int entry, int v) { return int_of_real(s_rows[entry * kSavedStride + kBackReals + v]); });
             wave_lds_sync();
         }
     }

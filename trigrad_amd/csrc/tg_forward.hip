@@ -55,6 +55,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
     publish_wave_rect(p, s_rects);
+    uint64_t *const masks = out.hit_masks ? out.hit_masks + hit_mask_head_words() : nullptr;
 
     PixelState s;
     int last = 0;
@@ -71,13 +72,13 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         uint64_t m[kBatch / kWave];
         batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
         if (!running) m[0] = m[1] = m[2] = m[3] = 0;
-        if (out.hit_masks) {
+        if (masks) {
             // kept for the backward pass, which then has no inside test to repeat
             const int64_t chunk = hit_mask_chunk(start, tile, batch - start);
             const int64_t slots = (int64_t)gridDim.z * blockDim.x, slot = (int64_t)blockIdx.z * blockDim.x + tid;
 #pragma unroll
             for (int wd = 0; wd < kBatch / kWave; wd++)
-                if (wd * kWave < nb) out.hit_masks[(chunk + wd) * slots + slot] = m[wd];
+                if (wd * kWave < nb) masks[(chunk + wd) * slots + slot] = m[wd];
         }
         // 2. every lane composites its own hits in list order, so the blend arithmetic
         //    runs with as many lanes busy as there are pixels with a fragment left
@@ -95,6 +96,19 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         }
     }
     if (p.valid) write_pixel(out, p, s, last, 0.0f);
+    if (out.hit_masks) {
+        // how far into the list this workgroup's pixels got
+        __shared__ int s_last;
+        __syncthreads();
+        if (tid == 0) s_last = 0;
+        __syncthreads();
+        int wave_last = p.valid ? last : 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) wave_last = max(wave_last, __shfl_xor(wave_last, off, kWave));
+        if ((tid & (kWave - 1)) == 0 && wave_last > 0) atomicMax(&s_last, wave_last);
+        __syncthreads();
+        if (tid == 0) out.hit_masks[hit_mask_head_index()] = (uint64_t)s_last;
+    }
 }
 
 // render.cu:338-373 insert_sorted_topk on an LDS candidate list of capacity `cap`.
@@ -307,7 +321,7 @@ extern "C" size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int t
     if (n_keys < 0 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0 || tile_w * tile_h > kMaxTilePixels) return 0;
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, kTileThreads);
     const int64_t tiles = (int64_t)tl.grid.x * tl.grid.y;
-    return (size_t)((n_keys / kWave + tiles + 1) * (int64_t)tl.grid.z * tl.threads);
+    return (size_t)(tiles * tl.grid.z + (n_keys / kWave + tiles + 1) * (int64_t)tl.grid.z * tl.threads);
 }
 
 extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, const real *colors, const real *opacities,

@@ -112,14 +112,20 @@ __device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRe
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
 }
 
-// Saved hit masks (tile order): word (chunk * slots + slot) holds, for the pixel
-// in thread slot `slot` of its tile, which of 64 consecutive list entries cover
-// it.  The chunks of a tile whose list starts at `start` are numbered from
-// start / 64 + tile: consecutive tiles never share a chunk, and
+// Saved hit masks (tile order).  The buffer starts with one word per workgroup of the tile launch
+// (index hit_mask_head_index()): the largest `last` among the workgroup's pixels, i.e. how much of the
+// list the backward pass has to walk, known to it without waiting for its pixels' loads.  Then, from
+// word hit_mask_head_words() on, word (chunk * slots + slot) holds, for the pixel in thread slot `slot`
+// of its tile, which of 64 consecutive list entries cover it.  The chunks of a tile whose list starts
+// at `start` are numbered from start / 64 + tile: consecutive tiles never share a chunk, and
 // n_keys / 64 + n_tiles + 1 chunks hold every list.
 __device__ __forceinline__ int64_t hit_mask_chunk(int start, int tile, int relative_position) {
     return (int64_t)(start >> 6) + tile + (relative_position >> 6);
 }
+__device__ __forceinline__ int64_t hit_mask_head_index() {
+    return ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * gridDim.z + blockIdx.z;
+}
+__device__ __forceinline__ int64_t hit_mask_head_words() { return (int64_t)gridDim.x * gridDim.y * gridDim.z; }
 
 // Batch bounds: word batch_bound_index(start, tile, p) holds, for the tile whose
 // list starts at `start`, a lower bound of the per-pixel depth of every entry at
