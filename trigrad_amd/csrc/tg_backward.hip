@@ -424,6 +424,22 @@ __device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads,
 
 __device__ __forceinline__ int top_bit(uint64_t m) { return 63 - __builtin_clzll(m); }
 
+// Transposes the 64 x 64 bit matrix whose row i is the word x of lane i: afterwards bit i of
+// lane b's word is what bit b of lane i's word was.  Six exchange steps between lanes 32, 16, ... 1
+// apart, each swapping the off-diagonal blocks of that size.
+__device__ __forceinline__ uint64_t transpose_bits(uint64_t x, int lane) {
+    constexpr uint64_t kHigh[6] = {0xFFFFFFFF00000000ull, 0xFFFF0000FFFF0000ull, 0xFF00FF00FF00FF00ull,
+                                   0xF0F0F0F0F0F0F0F0ull, 0xCCCCCCCCCCCCCCCCull, 0xAAAAAAAAAAAAAAAAull};
+#pragma unroll
+    for (int s = 0; s < 6; s++) {
+        const int j = 32 >> s;
+        const uint32_t lo = __shfl_xor((uint32_t)x, j, kWave), hi = __shfl_xor((uint32_t)(x >> 32), j, kWave);
+        const uint64_t y = ((uint64_t)hi << 32) | lo;
+        x = (lane & j) ? (x & kHigh[s]) | ((y >> j) & ~kHigh[s]) : (x & ~kHigh[s]) | ((y << j) & kHigh[s]);
+    }
+    return x;
+}
+
 __device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
     return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
@@ -535,29 +551,14 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
         // 1. which entries cover which pixel: read back what the forward pass saved, or test again
         //    (then only the entries that can touch this wave's pixels)
         if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
-        ballots[lane] = 0;
-        ballots[lane + kWave] = 0;
-        wave_lds_sync();
         if (saved_masks) {
-#pragma unroll
-            for (int wd = 0; wd < 2; wd++) {
-                const uint64_t bits = m[wd];
-                // per-entry ballots = the transpose, for the entries any lane holds
-                uint32_t any_lo = (uint32_t)bits, any_hi = (uint32_t)(bits >> 32);
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) {
-                    any_lo |= __shfl_xor(any_lo, off, kWave);
-                    any_hi |= __shfl_xor(any_hi, off, kWave);
-                }
-                uint64_t todo = ((uint64_t)any_hi << 32) | any_lo;
-                while (todo) {
-                    const int bit = __builtin_ctzll(todo);
-                    todo &= todo - 1;
-                    const uint64_t vote = __builtin_amdgcn_ballot_w64((bits >> bit) & 1);
-                    if (lane == 0) ballots[64 * wd + bit] = vote;
-                }
-            }
+            // per-entry ballots = the transpose of the lanes' masks
+            ballots[lane] = transpose_bits(m[0], lane);
+            ballots[lane + kWave] = transpose_bits(m[1], lane);
         } else {
+            ballots[lane] = 0;
+            ballots[lane + kWave] = 0;
+            wave_lds_sync();
 #pragma unroll
             for (int wd = 0; wd < 2; wd++) {
                 uint64_t bits = 0;
