@@ -324,8 +324,7 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
 
 
 constexpr int kBackBatch = 128;   // list entries staged per batch
-constexpr int kWaveSlots = 256;   // hit slots per wave and round
-constexpr int kSeedWords = 6;     // d_do, gc[3], dd_dz, (entry | source lane << 8)
+constexpr int kWaveSlots = 64;    // hit slots per wave and round: one per lane of the order-free part
 constexpr int kTermStride = 65;   // row stride of the per-wave term matrix (odd: conflict-free columns)
 constexpr int kMaxWaves = kTileThreads / kWave;
 
@@ -468,9 +467,8 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     __shared__ BackRecord s_rec[kBackBatch];
     __shared__ uint64_t s_ballot[kMaxWaves][kBackBatch];
     __shared__ uint32_t s_base[kMaxWaves][kBackBatch];
-    __shared__ real s_seed[kMaxWaves][kSeedWords][kWaveSlots];
+    __shared__ int s_tag[kMaxWaves][kWaveSlots];  // (entry | source lane << 8) of a slot
     __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
-    __shared__ real s_px[kTileThreads], s_py[kTileThreads];
     __shared__ uint8_t s_touch[kBackBatch];
     __shared__ WaveRect s_rects[kMaxTileWaves];
     __shared__ int s_last;
@@ -484,7 +482,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     const TermLane tl = term_lane<kLayout>(g, lane);
     uint64_t *ballots = s_ballot[wave];
     uint32_t *bases = s_base[wave];
-    real (*seeds)[kWaveSlots] = s_seed[wave];
+    int *tags = s_tag[wave];
     real *terms = s_term[wave];
 
     // With the forward pass's masks comes the number of list entries this workgroup has to walk; else
@@ -495,8 +493,6 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     const int my_last = p.valid ? g.last[p.index] : 0;  // entries [0, my_last) of the list may hold my fragments
     BackState st;
     if (p.valid) st = load_back_state(g, p);
-    s_px[tid] = p.px;
-    s_py[tid] = p.py;
     int tile_last;
     if (saved_masks) {
         tile_last = (int)g.hit_masks[hit_mask_head_index()];
@@ -614,47 +610,45 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                     real b0, b1, b2;
                     bary_apply(r.m, p.px, p.py, b0, b1, b2);
                     const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
-                    seeds[0][slot] = f.d_do;
-                    seeds[1][slot] = f.gc[0];
-                    seeds[2][slot] = f.gc[1];
-                    seeds[3][slot] = f.gc[2];
-                    seeds[4][slot] = f.dd_dz;
-                    seeds[5][slot] = int_in_real(e | (lane << 8));
+                    // the five numbers wait in the slot's column of the term matrix, which is free until
+                    // the slot's own lane replaces them by the terms
+                    terms[0 * kTermStride + slot] = f.d_do;
+                    terms[1 * kTermStride + slot] = f.gc[0];
+                    terms[2 * kTermStride + slot] = f.gc[1];
+                    terms[3 * kTermStride + slot] = f.gc[2];
+                    terms[4 * kTermStride + slot] = f.dd_dz;
+                    tags[slot] = e | (lane << 8);
                 }
             }
             wave_lds_sync();
 
-            // 4. order-free part
-            for (int s0 = 0; s0 < n_slots; s0 += kWave) {
-                const int n_here = min(kWave, n_slots - s0);
-                int tag = -1;
-                if (lane < n_here) {
-                    const int slot = s0 + lane;
-                    FragSeed f;
-                    f.d_do = seeds[0][slot];
-                    f.gc[0] = seeds[1][slot];
-                    f.gc[1] = seeds[2][slot];
-                    f.gc[2] = seeds[3][slot];
-                    f.dd_dz = seeds[4][slot];
-                    const int packed = int_of_real(seeds[5][slot]);
-                    tag = packed & 0xff;
-                    const int src = wave * kWave + (packed >> 8);
-                    const real px = s_px[src], py = s_py[src];
-                    const BackRecord &r = s_rec[tag];
-                    real b0, b1, b2;
-                    bary_apply(r.m, px, py, b0, b1, b2);
-                    real term[kTerms];
-                    fragment_terms(f, r, b0, b1, b2, px, py, term);
+            // 4. order-free part: lane = slot
+            int tag = -1;
+            if (lane < n_slots) tag = tags[lane] & 0xff;
+            // the pixel of the slot, from the lane that owns it
+            const int src = (lane < n_slots) ? tags[lane] >> 8 : lane;
+            const real px = __shfl(p.px, src, kWave), py = __shfl(p.py, src, kWave);
+            if (lane < n_slots) {
+                FragSeed f;
+                f.d_do = terms[0 * kTermStride + lane];
+                f.gc[0] = terms[1 * kTermStride + lane];
+                f.gc[1] = terms[2 * kTermStride + lane];
+                f.gc[2] = terms[3 * kTermStride + lane];
+                f.dd_dz = terms[4 * kTermStride + lane];
+                const BackRecord &r = s_rec[tag];
+                real b0, b1, b2;
+                bary_apply(r.m, px, py, b0, b1, b2);
+                real term[kTerms];
+                fragment_terms(f, r, b0, b1, b2, px, py, term);
 #pragma unroll
-                    for (int q = 0; q < kTerms; q++) terms[q * kTermStride + lane] = term[q];
-                }
-                const int tag_before = __shfl_up(tag, 1, kWave);
-                const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_here && (lane == 0 || tag != tag_before));
-                wave_lds_sync();
-                add_run_sums(terms, n_here, heads, tl, [&](int c) { return int_of_real(seeds[5][s0 + c]) & 0xff; },
-                             [&](int entry, int v) { return s_rec[entry].id[v]; });
-                wave_lds_sync();
+                for (int q = 0; q < kTerms; q++) terms[q * kTermStride + lane] = term[q];
             }
+            const int tag_before = __shfl_up(tag, 1, kWave);
+            const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tag != tag_before));
+            wave_lds_sync();
+            add_run_sums(terms, n_slots, heads, tl, [&](int c) { return tags[c] & 0xff; },
+                         [&](int entry, int v) { return s_rec[entry].id[v]; });
+            wave_lds_sync();
         }
     }
 }
