@@ -12,7 +12,7 @@
 //
 // per_pixel_sort = 0 (backward_tile_order_kernel): all pixels of a tile share
 //   the list order, so the tile's list is walked backwards in LDS-staged
-//   batches of 128 entries.
+//   batches of 64 entries.
 // per_pixel_sort = 1, max_layers <= 32 (backward_saved_order_kernel): every
 //   pixel walks the blend order the forward pass saved for it, backwards.
 // per_pixel_sort = 1, max_layers > 32 (backward_pixel_order_kernel): the pixel
@@ -323,7 +323,8 @@ __device__ __forceinline__ BackState load_back_state(const BackwardArgs &g, cons
 }
 
 
-constexpr int kBackBatch = 128;   // list entries staged per batch
+constexpr int kBackBatch = 64;    // list entries staged per batch
+constexpr int kBackWords = kBackBatch / kWave;  // words of a lane's hit mask per batch
 constexpr int kWaveSlots = 64;    // hit slots per wave and round: one per lane of the order-free part
 constexpr int kTermStride = 65;   // row stride of the per-wave term matrix (odd: conflict-free columns)
 constexpr int kMaxWaves = kTileThreads / kWave;
@@ -445,23 +446,25 @@ __device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
 
 // Tile-order backward.  LDS floating-point atomics cost about three cycles per lane on
 // gfx950 and direct global atomics collide on the shared vertices, so the
-// per-entry sums are formed with plain LDS stores and loads.  The records of
-// 128 list entries are staged per batch by the whole workgroup; after that
-// every wave works on its own 64 pixels without workgroup barriers:
-//   1. every lane tests its pixel against every record (same record for all
-//      lanes: LDS broadcast) and keeps its hits as a 128-bit mask; the wave's
-//      ballot per record is stored;
+// per-entry sums are formed with plain LDS stores and loads.  The kernel is bound by
+// latency (LDS round trips, dependent loads), so its LDS and register budgets are set
+// for four workgroups per CU: the records of 64 list entries are staged per batch by
+// the whole workgroup; after that every wave works on its own 64 pixels without
+// workgroup barriers:
+//   1. which entries cover which pixel: the lane's 64-bit mask the forward pass saved
+//      (or the inside tests again, same record for all lanes: LDS broadcast); the
+//      wave's ballot per entry is the transpose of the lanes' masks;
 //   2. the ballots become slot numbers: entries from the far end, lanes in
 //      order inside an entry, so every (pixel, entry) hit of the wave owns one
 //      slot, slots are grouped by entry, and a lane's own hits have increasing
 //      numbers in the order it must visit them (reverse blend order);
-//   3. ordered part, in rounds of 256 slots: every lane walks its own hits and
+//   3. ordered part, in rounds of 64 slots: every lane walks its own hits and
 //      advances the pixel's transmittance and running sums; each hit leaves
 //      five numbers in its slot;
-//   4. order-free part, 64 slots at a time with every lane busy: lane = slot
-//      evaluates the 21 gradient terms of its hit and writes them to a term
-//      matrix; three groups of 21 lanes add up the runs of equal entry and issue
-//      one global floating-point atomic per run and term.
+//   4. order-free part with every lane busy: lane = slot evaluates the 21 gradient
+//      terms of its hit and writes them to a term matrix; three groups of 21 lanes
+//      add up the runs of equal entry and issue one global floating-point atomic
+//      per run and term.
 template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ BackRecord s_rec[kBackBatch];
@@ -506,41 +509,28 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     }
 
     // Batches are aligned to multiples of kBackBatch from the start of the list (the last one may be
-    // short), so that a batch is two whole words of the saved hit masks.
+    // short), so that a batch is whole words of the saved hit masks.
     const int64_t mask_slots = (int64_t)gridDim.z * blockDim.x, mask_slot = (int64_t)blockIdx.z * blockDim.x + tid;
-    // A workgroup with a thread per staged entry keeps the entry of the next batch in registers: its
-    // loads are issued when a batch starts and land in LDS when the next one does.
-    const bool ahead = (int)blockDim.x >= kBackBatch;
     const int hi0 = (tile_last + kBackBatch - 1) / kBackBatch * kBackBatch;
-    BackRecord next;
-    if (ahead && hi0 > 0 && tid < tile_last - (hi0 - kBackBatch)) gather_back(a, start + hi0 - kBackBatch + tid, next);  // hi0 = 0: nothing to walk
     for (int hi = hi0; hi > 0; hi -= kBackBatch) {
         const int lo = hi - kBackBatch;
         const int nb = min(hi, tile_last) - lo;
         const int mine = my_last - lo;  // records [0, mine) of this batch are within my range
         // my saved masks of the batch: asked for here, used after the staging
-        uint64_t m[2] = {0, 0};
+        uint64_t m[kBackWords] = {};
         if (saved_masks) {
             const int64_t chunk = hit_mask_chunk(start, tile, lo);
 #pragma unroll
-            for (int wd = 0; wd < 2; wd++)
+            for (int wd = 0; wd < kBackWords; wd++)
                 if (64 * wd < mine) {
                     m[wd] = masks[(chunk + wd) * mask_slots + mask_slot];
                     if (mine < 64 * wd + 64) m[wd] &= (1ull << (mine - 64 * wd)) - 1;  // entries past my last one
                 }
         }
         __syncthreads();  // every wave is done with the previous batch
-        if (ahead) {
-            if (tid < nb) {
-                s_rec[tid] = next;
-                if (!saved_masks) s_touch[tid] = (uint8_t)waves_touched(next.m, s_rects, n_waves);
-            }
-            if (lo > 0 && tid < kBackBatch) gather_back(a, start + lo - kBackBatch + tid, next);  // all batches but the first are full
-        } else {
-            for (int e = tid; e < nb; e += blockDim.x) {
-                gather_back(a, start + lo + e, s_rec[e]);
-                if (!saved_masks) s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
-            }
+        for (int e = tid; e < nb; e += blockDim.x) {
+            gather_back(a, start + lo + e, s_rec[e]);
+            if (!saved_masks) s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
         }
         __syncthreads();
 
@@ -549,14 +539,14 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
         if (__builtin_amdgcn_ballot_w64(mine > 0) == 0) continue;  // nothing for this wave in the batch
         if (saved_masks) {
             // per-entry ballots = the transpose of the lanes' masks
-            ballots[lane] = transpose_bits(m[0], lane);
-            ballots[lane + kWave] = transpose_bits(m[1], lane);
+#pragma unroll
+            for (int wd = 0; wd < kBackWords; wd++) ballots[wd * kWave + lane] = transpose_bits(m[wd], lane);
         } else {
-            ballots[lane] = 0;
-            ballots[lane + kWave] = 0;
+#pragma unroll
+            for (int wd = 0; wd < kBackWords; wd++) ballots[wd * kWave + lane] = 0;
             wave_lds_sync();
 #pragma unroll
-            for (int wd = 0; wd < 2; wd++) {
+            for (int wd = 0; wd < kBackWords; wd++) {
                 uint64_t bits = 0;
                 uint64_t todo = wave_candidates(s_touch, 64 * wd, nb, wave);
                 while (todo) {
@@ -578,14 +568,22 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
         // 2. slot numbers of this wave
         uint32_t n_hits;
         {
-            uint32_t cnt[2];
-            const int e0 = nb - 1 - 2 * lane, e1 = e0 - 1;
-            cnt[0] = e0 >= 0 ? (uint32_t)__builtin_popcountll(ballots[e0]) : 0u;
-            cnt[1] = e1 >= 0 ? (uint32_t)__builtin_popcountll(ballots[e1]) : 0u;
-            const uint32_t incl = wave_inclusive_scan_u32(cnt[0] + cnt[1]);
-            const uint32_t excl = incl - cnt[0] - cnt[1];
-            if (e0 >= 0) bases[e0] = excl;
-            if (e1 >= 0) bases[e1] = excl + cnt[0];
+            // lane l takes entries nb - 1 - kBackWords * l and the kBackWords - 1 before it
+            uint32_t cnt[kBackWords], mine_total = 0;
+#pragma unroll
+            for (int k = 0; k < kBackWords; k++) {
+                const int e = nb - 1 - kBackWords * lane - k;
+                cnt[k] = e >= 0 ? (uint32_t)__builtin_popcountll(ballots[e]) : 0u;
+                mine_total += cnt[k];
+            }
+            const uint32_t incl = wave_inclusive_scan_u32(mine_total);
+            uint32_t base = incl - mine_total;
+#pragma unroll
+            for (int k = 0; k < kBackWords; k++) {
+                const int e = nb - 1 - kBackWords * lane - k;
+                if (e >= 0) bases[e] = base;
+                base += cnt[k];
+            }
             n_hits = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
         }
         wave_lds_sync();
@@ -596,8 +594,9 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
             while (true) {
                 int e = -1;
                 uint32_t slot = 0;
-                if (m[1]) e = 64 + top_bit(m[1]);
-                else if (m[0]) e = top_bit(m[0]);
+#pragma unroll
+                for (int wd = kBackWords - 1; wd >= 0; wd--)
+                    if (e < 0 && m[wd]) e = 64 * wd + top_bit(m[wd]);
                 if (e >= 0) {
                     slot = bases[e] + lanes_below_mask(ballots[e]) - round0;
                     if (slot >= (uint32_t)kWaveSlots) e = -1;
@@ -605,7 +604,9 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
                 const bool active = e >= 0;
                 if (__builtin_amdgcn_ballot_w64(active) == 0) break;
                 if (active) {
-                    if (e >= 64) m[1] &= ~(1ull << (e - 64)); else m[0] &= ~(1ull << e);
+#pragma unroll
+                    for (int wd = 0; wd < kBackWords; wd++)
+                        if ((e >> 6) == wd) m[wd] &= ~(1ull << (e & 63));
                     const BackRecord &r = s_rec[e];
                     real b0, b1, b2;
                     bary_apply(r.m, p.px, p.py, b0, b1, b2);
