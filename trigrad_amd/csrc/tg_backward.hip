@@ -365,11 +365,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 // gradient arrays.  Bit c of `heads` is set where slot c starts a run.  First every lane (group, q)
 // turns its third of row q into running sums that start over at each head: no branch and no look at
 // the entries.  The last slot of a run, and of a third, then holds a sum to deliver; those slots are
-// taken three at a time, one per group.  entry_at(c): list entry of slot c; vertex_of(entry, v):
-// vertex id v of that entry.
-template <typename EntryAt, typename VertexOf>
-__device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads, const TermLane &t, EntryAt entry_at,
-                                             VertexOf vertex_of) {
+// taken three at a time, one per group.  vertex_at(c, v): vertex id v of the entry in slot c.
+template <typename VertexAt>
+__device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads, const TermLane &t, VertexAt vertex_at) {
     constexpr int kAhead = 8;  // terms read ahead, so that the LDS latency is paid once per eight slots
     const int per = (n + 2) / 3;
     const int c0 = min(t.group * per, n), c1 = min(c0 + per, n);
@@ -406,16 +404,13 @@ __device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads,
                     if (t.group == k) c[u] = bit;
                 }
         real sum[2] = {0.0f, 0.0f};
-        int entry[2] = {0, 0}, vertex[2] = {0, 0};
+        int vertex[2] = {0, 0};
 #pragma unroll
         for (int u = 0; u < 2; u++)
             if (c[u] >= 0) {
                 sum[u] = row[c[u]];
-                entry[u] = entry_at(c[u]);
+                vertex[u] = vertex_at(c[u], t.vertex);
             }
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-            if (c[u] >= 0) vertex[u] = vertex_of(entry[u], t.vertex);
 #pragma unroll
         for (int u = 0; u < 2; u++)
             if (sum[u] != 0.0f) unsafeAtomicAdd(t.base + (int64_t)t.stride * vertex[u], sum[u]);
@@ -647,8 +642,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
             const int tag_before = __shfl_up(tag, 1, kWave);
             const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tag != tag_before));
             wave_lds_sync();
-            add_run_sums(terms, n_slots, heads, tl, [&](int c) { return tags[c] & 0xff; },
-                         [&](int entry, int v) { return s_rec[entry].id[v]; });
+            add_run_sums(terms, n_slots, heads, tl, [&](int c, int v) { return s_rec[tags[c] & 0xff].id[v]; });
             wave_lds_sync();
         }
     }
@@ -780,45 +774,32 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 }
 
 // Per-pixel order with the blend order saved by the forward pass
-// (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  The records of the first
-// kSavedWindow list entries of the tile are staged once (rows an odd number of
-// words apart, so lanes reading different entries use different banks).  Every
-// wave walks its 64 pixels in lockstep, each lane from its own far end.  LDS
-// floating-point atomics cost about three cycles per lane on gfx950 and many lanes of a
-// wave hold the same entry in the same step, so the 21 gradient terms of a step
-// are grouped by entry first: lanes with equal entries get consecutive slots
-// (ballot matching, groups in order of their lowest lane), the terms go to a
-// slot-major matrix in LDS, three groups of 21 lanes add up the runs of equal
-// entry and issue one global floating-point atomic per run and term.  Fragments of
-// entries beyond the staged window are gathered from and added to memory
-// directly.
-constexpr int kSavedWindow = 256;
-constexpr int kSavedStride = kBackReals + 3;  // 36 scalars, 3 vertex ids; odd
-
+// (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  Every wave walks its 64
+// pixels in lockstep, each lane from its own far end; a lane gathers the record of
+// its fragment from memory (neighbouring pixels hold the same few entries, so the
+// loads hit in cache; staging the tile's records in LDS first was measured slower,
+// for the workgroups per CU it costs).  LDS floating-point atomics cost about three
+// cycles per lane on gfx950 and many lanes of a wave hold the same entry in the same
+// step, so the 21 gradient terms of a step are grouped by entry first: lanes with
+// equal entries get consecutive slots (ballot matching, groups in order of their
+// lowest lane), the terms go to a slot-major matrix in LDS, three groups of 21 lanes
+// add up the runs of equal entry and issue one global floating-point atomic per run
+// and term.
 template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
-    __shared__ real s_rows[kSavedWindow * kSavedStride];
     __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
     __shared__ int s_tag[kMaxWaves][kWave];
+    __shared__ int s_vertex[kMaxWaves][3 * kWave];  // the three vertex ids of a slot's entry
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a);
-    const int n_win = min(end - start, kSavedWindow);
-    for (int e = tid; e < n_win; e += blockDim.x) {
-        BackRecord r;
-        gather_back(a, start + e, r);
-        const real *w = reinterpret_cast<const real *>(&r);
-#pragma unroll
-        for (int k = 0; k < kBackReals; k++) s_rows[e * kSavedStride + k] = w[k];
-#pragma unroll
-        for (int k = 0; k < 3; k++) s_rows[e * kSavedStride + kBackReals + k] = int_in_real(r.id[k]);
-    }
-    __syncthreads();
+    const int rel_bits = 32 - __builtin_clz(max(end - start - 1, 1));  // bits that tell two list positions apart
     real *terms = s_term[wave];
     int *tags = s_tag[wave];
+    int *vertices = s_vertex[wave];
     const TermLane tl = term_lane<kLayout>(g, lane);
 
     BackState st;
@@ -841,52 +822,39 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
         for (int u = 0; u < kGatherAhead; u++) {
             if (s0 + u >= n_max) break;  // wave-uniform
             const bool active = s0 + u < n;
-            const bool staged = active && rel[u] < n_win;
             real term[kTerms];
+            BackRecord r;
             if (active) {
-                BackRecord r;
-                if (staged) {
-                    real *w = reinterpret_cast<real *>(&r);
-#pragma unroll
-                    for (int k = 0; k < kBackReals; k++) w[k] = s_rows[rel[u] * kSavedStride + k];
-                } else {
-                    gather_back(a, start + rel[u], r);
-                }
+                gather_back(a, start + rel[u], r);
                 real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
-                if (!staged) {
-#pragma unroll
-                    for (int q = 0; q < kTerms; q++)
-                        if (term[q] != 0.0f) unsafeAtomicAdd(term_address<kLayout>(g, r.id[q / 7], q % 7), term[q]);
-                }
             }
             // slots: lanes with the same entry next to each other, groups in order of their lowest lane
-            uint64_t peers = __builtin_amdgcn_ballot_w64(staged);
-            if (peers == 0) continue;  // wave-uniform
-#pragma unroll
-            for (int b = 0; b < 8; b++) {
+            uint64_t peers = __builtin_amdgcn_ballot_w64(active);
+            for (int b = 0; b < rel_bits; b++) {  // wave-uniform
                 const bool bit = (rel[u] >> b) & 1;
                 const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
                 peers &= bit ? vote : ~vote;
             }
             const uint32_t rank = lanes_below_mask(peers);
-            const bool leads = staged && rank == 0;
+            const bool leads = active && rank == 0;
             const uint32_t size = leads ? (uint32_t)__builtin_popcountll(peers) : 0u;
             const uint32_t incl = wave_inclusive_scan_u32(size);
             const int n_slots = __builtin_amdgcn_readlane((int)incl, kWave - 1);
-            const int leader = staged ? __builtin_ctzll(peers) : lane;
+            const int leader = active ? __builtin_ctzll(peers) : lane;
             const int slot = __shfl((int)(incl - size), leader, kWave) + (int)rank;
-            if (staged) {
+            if (active) {
 #pragma unroll
                 for (int q = 0; q < kTerms; q++) terms[q * kTermStride + slot] = term[q];
                 tags[slot] = rel[u];
+#pragma unroll
+                for (int k = 0; k < 3; k++) vertices[k * kWave + slot] = r.id[k];
             }
             wave_lds_sync();
             // a slot starts a run where its entry differs from the slot before
             const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tags[lane] != tags[max(lane - 1, 0)]));
-            add_run_sums(terms, n_slots, heads, tl, [&](int c) { return tags[c]; },
-                         [&](int entry, int v) { return int_of_real(s_rows[entry * kSavedStride + kBackReals + v]); });
+            add_run_sums(terms, n_slots, heads, tl, [&](int c, int v) { return vertices[v * kWave + c]; });
             wave_lds_sync();
         }
     }
