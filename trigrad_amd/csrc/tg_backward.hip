@@ -719,10 +719,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
             }
             __syncthreads();
             uint64_t m[kBatch / kWave];
-            batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
+            batch_hit_mask<kBatch / kWave>(s_rec, s_touch, nb, wave, p.px, p.py, m);
             if (!want) m[0] = m[1] = m[2] = m[3] = 0;
             while (true) {
-                const int e = pop_lowest(m);
+                const int e = pop_lowest<kBatch / kWave>(m);
                 if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
                 if (e < 0) continue;
                 const DepthRecord &r = s_rec[e];
@@ -860,7 +860,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     }
 }
 
-size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads) + (size_t)kAccWindow * kTerms * sizeof(real); }
+size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads, kBatch) + (size_t)kAccWindow * kTerms * sizeof(real); }
 
 }  // namespace tg
 

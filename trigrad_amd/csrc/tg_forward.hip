@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         __syncthreads();
         // 1. inside tests; a lane keeps its hits as a 256-bit mask
         uint64_t m[kBatch / kWave];
-        batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
+        batch_hit_mask<kBatch / kWave>(s_rec, s_touch, nb, wave, p.px, p.py, m);
         if (!running) m[0] = m[1] = m[2] = m[3] = 0;
         if (masks) {
             // kept for the backward pass, which then has no inside test to repeat
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         //    runs with as many lanes busy as there are pixels with a fragment left
         while (true) {
             int e = -1;
-            if (s.alpha > a.thr && s.blended < a.max_layers) e = pop_lowest(m);  // render.cu:578, tested before every fragment
+            if (s.alpha > a.thr && s.blended < a.max_layers) e = pop_lowest<kBatch / kWave>(m);  // render.cu:578, tested before every fragment
             if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
             if (e >= 0) {
                 const BlendRecord &r = s_rec[e];
@@ -125,16 +125,19 @@ __device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, rea
     if (n < cap) n++;
 }
 
+constexpr int kSelectBatch = 128;
+
+template <int kStage>  // list entries staged per batch
 __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(RasterArgs a, ForwardOut out) {
     extern __shared__ __align__(16) unsigned char s_dyn[];
     const int n_threads = blockDim.x;
     DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
     TopK tk;
-    tk.depth = reinterpret_cast<real *>(s_dyn + sizeof(DepthRecord) * kBatch);
+    tk.depth = reinterpret_cast<real *>(s_dyn + sizeof(DepthRecord) * kStage);
     tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
 
-    __shared__ uint8_t s_touch[kBatch];
+    __shared__ uint8_t s_touch[kStage];
     __shared__ WaveRect s_rects[kMaxTileWaves];
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
@@ -153,8 +156,8 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         if (!__syncthreads_or(want)) break;
         const int cap = want ? min(kLayers, a.max_layers - s.blended) : 0;
         int found = 0;
-        for (int batch = start; batch < end; batch += kBatch) {
-            const int nb = min(kBatch, end - batch);
+        for (int batch = start; batch < end; batch += kStage) {
+            const int nb = min(kStage, end - batch);
             if (a.batch_bounds) {
                 // a lane needs nothing from here on when its list is full and its worst candidate is nearer than
                 // every fragment the rest of the tile's list can produce (a full list rejects depths >= its worst)
@@ -162,9 +165,9 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 const bool settled = !want || (found == cap && tk.d(cap - 1) <= rest);
                 if (__syncthreads_and(settled)) {
                     // on to the batch that holds the first entry the bounds do not cover
-                    const int resume = start + a.far_start[tile] / kBatch * kBatch;
+                    const int resume = start + a.far_start[tile] / kStage * kStage;
                     if (resume > batch) {
-                        batch = resume - kBatch;
+                        batch = resume - kStage;
                         continue;
                     }
                 }
@@ -177,11 +180,14 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
             __syncthreads();
             // inside tests into a per-lane mask, then every lane visits its own hits in
             // list order (the order insert_sorted_topk sees them in the reference)
-            uint64_t m[kBatch / kWave];
-            batch_hit_mask(s_rec, s_touch, nb, wave, p.px, p.py, m);
-            if (!want) m[0] = m[1] = m[2] = m[3] = 0;
+            uint64_t m[kStage / kWave];
+            batch_hit_mask<kStage / kWave>(s_rec, s_touch, nb, wave, p.px, p.py, m);
+            if (!want) {
+#pragma unroll
+                for (int wd = 0; wd < kStage / kWave; wd++) m[wd] = 0;
+            }
             while (true) {
-                const int e = pop_lowest(m);
+                const int e = pop_lowest<kStage / kWave>(m);
                 if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform
                 if (e < 0) continue;
                 const DepthRecord &r = s_rec[e];
@@ -203,7 +209,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         const real todo_depth = todo > 0 ? tk.d(todo - 1) : 0.0f;
         __syncthreads();
         real *rows = reinterpret_cast<real *>(s_dyn);
-        const int n_rows = min(end - start, (int)((sizeof(DepthRecord) * kBatch + sizeof(real) * kLayers * n_threads) /
+        const int n_rows = min(end - start, (int)((sizeof(DepthRecord) * kStage + sizeof(real) * kLayers * n_threads) /
                                                    (sizeof(real) * kBlendWords)));
         for (int e = tid; e < n_rows; e += blockDim.x) {
             BlendRecord r;
@@ -262,13 +268,15 @@ TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_th
 }
 
 // Workgroup size of the per-pixel-sort kernels.  Their candidate lists take
-// 32 * (scalar + int) bytes of LDS per thread.  The forward kernel runs a
-// 16x16 tile as two workgroups of 128 threads that walk the same list: each
-// needs 47 KB, three fit a CU, and two waves meet at a barrier instead of four
-// (measured 22 to 34 % faster than one workgroup of 256 on the five
-// configurations, although every list entry is staged twice).  The re-selecting
-// backward kernel also keeps 43 KB of gradient sums and stays at 256 threads.
-// TRIGRAD_PIXEL_ORDER_THREADS (64, 128 or 256) overrides both.
+// 32 * (scalar + int) bytes of LDS per thread: 64 KB for the 256 threads of a
+// 16x16 tile.  The selection kernels are bound by latency, so what counts is
+// how many waves a CU holds: the forward kernel stages 128 list entries at a
+// time (7.5 KB), two workgroups of 256 threads fit a CU.  Measured on the five
+// configurations against 64, 192 and 256 staged entries and against tiles split
+// over two workgroups of 128 threads or four of 64 (which stage every entry two
+// or four times): 15 to 35 % faster than 256 entries and 128 threads.  The
+// re-selecting backward kernel also keeps 43 KB of gradient sums.
+// TRIGRAD_PIXEL_ORDER_THREADS (64, 128 or 256) overrides the workgroup size.
 int pixel_order_threads(int preferred) {
     static int override = -1;
     if (override < 0) {
@@ -281,8 +289,8 @@ int pixel_order_threads(int preferred) {
     return override ? override : preferred;
 }
 
-size_t pixel_order_lds_bytes(int n_threads) {
-    return sizeof(DepthRecord) * kBatch + (size_t)kLayers * n_threads * (sizeof(real) + sizeof(int));
+size_t pixel_order_lds_bytes(int n_threads, int staged_entries) {
+    return sizeof(DepthRecord) * staged_entries + (size_t)kLayers * n_threads * (sizeof(real) + sizeof(int));
 }
 
 // Dynamic LDS beyond 64 KB has to be enabled per kernel once.
@@ -351,7 +359,7 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         return TG_E_ARG;
     }
     ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments, per_pixel_sort ? nullptr : hit_masks};
-    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads(128) : kTileThreads);
+    const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads(kTileThreads) : kTileThreads);
     const dim3 grid = tl.grid;
     const int n_threads = tl.threads;
     hipStream_t s = (hipStream_t)stream;
@@ -359,9 +367,9 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         TG_LAUNCH(forward_tile_order_kernel, grid, dim3(n_threads), 0, s, a, o);
         return check_launch("forward_tile_order_kernel");
     }
-    const size_t lds = pixel_order_lds_bytes(n_threads);
+    const size_t lds = pixel_order_lds_bytes(n_threads, kSelectBatch);
     static size_t lds_reserved = 0;
-    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel, lds, &lds_reserved)) return e;
-    TG_LAUNCH(forward_pixel_order_kernel, grid, dim3(n_threads), lds, s, a, o);
+    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatch>, lds, &lds_reserved)) return e;
+    TG_LAUNCH_AS("forward_pixel_order_kernel", forward_pixel_order_kernel<kSelectBatch>, grid, dim3(n_threads), lds, s, a, o);
     return check_launch("forward_pixel_order_kernel");
 }

@@ -166,7 +166,7 @@ __device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord 
 struct TileLaunch { dim3 grid; int threads; };
 TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads);
 int pixel_order_threads(int preferred);
-size_t pixel_order_lds_bytes(int n_threads);
+size_t pixel_order_lds_bytes(int n_threads, int staged_entries);
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
 int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
 
@@ -241,11 +241,11 @@ __device__ __forceinline__ uint64_t wave_candidates(const uint8_t *s_touch, int 
 // result (word e / 64) is set when record e covers the pixel.  All lanes of the
 // wave read the same record at the same time (LDS broadcast); only records that
 // can touch the wave's pixels are looked at.  Rec must have a member m[9].
-template <typename Rec>
+template <int kWords, typename Rec>
 __device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *s_touch, int nb, int wave, real px, real py,
-                                               uint64_t m[kBatch / kWave]) {
+                                               uint64_t m[kWords]) {
 #pragma unroll
-    for (int wd = 0; wd < kBatch / kWave; wd++) {
+    for (int wd = 0; wd < kWords; wd++) {
         uint64_t bits = 0;
         uint64_t todo = wave_candidates(s_touch, wd * kWave, nb, wave);
         while (todo) {
@@ -259,14 +259,16 @@ __device__ __forceinline__ void batch_hit_mask(const Rec *s_rec, const uint8_t *
     }
 }
 
-// Lowest set bit of a 256-bit mask, removed from the mask; -1 if the mask is empty.
-__device__ __forceinline__ int pop_lowest(uint64_t m[kBatch / kWave]) {
-    static_assert(kBatch / kWave == 4, "four 64-bit words");
+// Lowest set bit of a mask of kWords 64-bit words, removed from the mask; -1 if the mask is empty.
+template <int kWords>
+__device__ __forceinline__ int pop_lowest(uint64_t m[kWords]) {
     int e = -1;
-    if (m[0]) { e = __builtin_ctzll(m[0]); m[0] &= m[0] - 1; }
-    else if (m[1]) { e = 64 + __builtin_ctzll(m[1]); m[1] &= m[1] - 1; }
-    else if (m[2]) { e = 128 + __builtin_ctzll(m[2]); m[2] &= m[2] - 1; }
-    else if (m[3]) { e = 192 + __builtin_ctzll(m[3]); m[3] &= m[3] - 1; }
+#pragma unroll
+    for (int wd = 0; wd < kWords; wd++)
+        if (e < 0 && m[wd]) {
+            e = 64 * wd + __builtin_ctzll(m[wd]);
+            m[wd] &= m[wd] - 1;
+        }
     return e;
 }
 
