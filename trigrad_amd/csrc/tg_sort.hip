@@ -76,8 +76,12 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
     for (; i < n_words; i += stride) p[i] = 0;
 }
 
+// Also clears `zero_words` words from `zero` on (the tickets and look-back words of the sweeps that
+// follow), a slice per workgroup: a launch of its own for that costs more than the stores.
 __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, int passes,
-                                                                      uint32_t *__restrict__ partials) {
+                                                                      uint32_t *__restrict__ partials, uint32_t *__restrict__ zero,
+                                                                      size_t zero_words) {
+    for (size_t i = (size_t)blockIdx.x * kSortThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kSortThreads) zero[i] = 0;
     // one set of counters per wave: the upper passes see few distinct digits (the tile bits), and LDS
     // atomics to one address serialise
     __shared__ uint32_t s_hist_wave[kSortWaves][kMaxPasses][kRadix];
@@ -353,11 +357,7 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
 
     // tickets and look-back words (adjacent) start at zero; bases and partials are fully overwritten
     const size_t fill_words = 64 + (size_t)L.passes * L.n_tiles * kRadix;
-    const int fill_blocks = (int)((fill_words + 1023) / 1024 < 2048 ? (fill_words + 1023) / 1024 : 2048);
-    TG_LAUNCH(fill_zero_kernel, dim3(fill_blocks), dim3(256), 0, s, tickets, fill_words);
-    if (int e = check_launch("fill_zero_kernel")) return e;
-
-    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials);
+    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials, tickets, fill_words);
     if (int e = check_launch("sort_histogram_kernel")) return e;
     TG_LAUNCH(sort_bases_kernel, dim3(L.passes), dim3(kBasesThreads), 0, s, partials, L.hist_blocks, bases, status);
     if (int e = check_launch("sort_bases_kernel")) return e;
