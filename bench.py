@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of sort_sweep_kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
 # 256 MiB plain copy (profiles/config2_hbm_traffic_counters.md), keyed by the number of pairs it was measured on.
-MEASURED_SWEEP_TRAFFIC = {2186877: 64.1e6}
+MEASURED_SWEEP_TRAFFIC = {2186877: 64.2e6}
 
 MODES = {
     "A": dict(per_pixel_sort=True, max_layers=32),    # API defaults
