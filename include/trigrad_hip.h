@@ -174,8 +174,10 @@ int tg_list_bounds(const tg_real *vertices, int32_t n_vertices, const int32_t *i
  * fragments again (the reference re-selects, render.cu:667-693).
  * hit_masks (tg_hit_mask_words() uint64 words), or NULL: without per_pixel_sort
  * the kernel also writes, for every pixel and every 64 consecutive entries of
- * its tile's list that it looked at, which of them cover the pixel;
- * tg_render_backward then reads them back instead of repeating the inside tests.
+ * its tile's list that it looked at, which of them cover the pixel, and per
+ * workgroup how far into the list its pixels got; tg_render_backward then
+ * reads them back instead of repeating the inside tests.  The buffer is
+ * private to the two calls: its layout is theirs to change.
  * batch_bounds, far_start: tg_list_bounds' outputs, or NULL (used with per_pixel_sort only).
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
 size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int tile_w, int tile_h);
