@@ -43,7 +43,17 @@ struct PixelCoord {
 __device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
     PixelCoord p;
     const int t = blockIdx.z * blockDim.x + threadIdx.x;
-    const int lx = t % a.tw, ly = t / a.tw;
+    int lx, ly;
+    if (((a.tw | a.th) & 7) == 0) {
+        // a wave takes a square of 8 x 8 pixels: fewer list entries touch a square than a strip of the
+        // same area, so the waves cull more and share an entry among more lanes
+        const int squares_x = a.tw >> 3, square = t >> 6, l = t & 63;
+        lx = (square % squares_x) * 8 + (l & 7);
+        ly = (square / squares_x) * 8 + (l >> 3);
+    } else {
+        lx = t % a.tw;
+        ly = t / a.tw;
+    }
     p.ix = blockIdx.x * a.tw + lx;
     p.iy = blockIdx.y * a.th + ly;
     p.valid = (t < a.tw * a.th) && p.ix < a.W && p.iy < a.H;  // render.cu:554
