@@ -32,16 +32,18 @@ int check_launch(const char *what) {
 // ---- per-kernel timing ---------------------------------------------------------
 struct ProfileRecord {
     const char *name;
+    int launches;
     hipEvent_t start, stop;
 };
 static bool g_profile_on = false;
 static std::mutex g_profile_mutex;
 static std::vector<ProfileRecord> g_profile_records;
 
-ProfileScope::ProfileScope(const char *name, hipStream_t s) : slot(-1), stream(s) {
+ProfileScope::ProfileScope(const char *name, hipStream_t s, int launches) : slot(-1), stream(s) {
     if (!g_profile_on) return;
     ProfileRecord r;
     r.name = name;
+    r.launches = launches;
     if (hipEventCreate(&r.start) != hipSuccess) return;
     if (hipEventCreate(&r.stop) != hipSuccess) { (void)hipEventDestroy(r.start); return; }
     (void)hipEventRecord(r.start, s);
@@ -101,7 +103,7 @@ extern "C" int tg_profile_report(char *buffer, size_t capacity) {
         float ms = 0.0f;
         if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
             Sum &s = sums[r.name];
-            s.count++;
+            s.count += r.launches;
             s.ms += ms;
         }
         (void)hipEventDestroy(r.start);

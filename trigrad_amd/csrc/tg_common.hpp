@@ -46,7 +46,7 @@ int check_launch(const char *what);
 // bracketed by a pair of events on its stream; tg_profile_report waits for
 // them and sums the elapsed time per kernel name.
 struct ProfileScope {
-    ProfileScope(const char *name, hipStream_t stream);
+    ProfileScope(const char *name, hipStream_t stream, int launches = 1);  // launches: kernels of that name inside the pair
     ~ProfileScope();
     int slot;
     hipStream_t stream;
