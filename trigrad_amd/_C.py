@@ -304,7 +304,7 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             arrived.synchronize()
         else:
             host = total._base.cpu()
-        K, st = int(host[0]), int(host[1])
+        K, st = host.tolist()  # one conversion: the device waits for the launches that follow
         if st != 0:
             raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
         keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
