@@ -97,7 +97,7 @@ def _grad_inputs(scene, seed, with_depth):
 
 
 BACKWARD_SCENES = ["config0", "soup_varying_w", "soup_shared", "soup_big_tris", "soup_tile4", "soup_tile32", "soup_tile_8x4",
-                   "squares", "large_triangles", "depth_overlap", "unit_square_negative_z", "grid_mesh", "degenerate", "center_island"]
+                   "squares", "large_triangles", "depth_overlap", "unit_square_negative_z", "grid_mesh", "degenerate", "center_island", "soup_tile8", "soup_tile_24x16"]
 
 
 @pytest.mark.parametrize("with_depth", [False, True])

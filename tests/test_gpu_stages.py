@@ -22,6 +22,8 @@ def _scenes():
         "soup_tile32": lambda: (S.random_soup(800, 200, 150, seed=5, sigma_px=12.0), 32, 32),
         "soup_tile_8x4": lambda: (S.random_soup(800, 100, 90, seed=6, sigma_px=7.0), 8, 4),
         "soup_tile_12x20": lambda: (S.random_soup(800, 130, 170, seed=7, sigma_px=7.0), 12, 20),
+        "soup_tile8": lambda: (S.random_soup(600, 90, 70, seed=8, sigma_px=6.0), 8, 8),            # one wave per tile
+        "soup_tile_24x16": lambda: (S.random_soup(800, 150, 110, seed=9, sigma_px=9.0), 24, 16),   # six 8x8 squares over two workgroups
         "squares": lambda: (S.overlapping_squares(10), 4, 4),
         "large_triangles": lambda: (S.large_triangles(3, r=4), 4, 4),
         "depth_overlap": lambda: (S.depth_overlap(), 16, 16),
