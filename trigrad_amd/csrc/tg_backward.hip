@@ -720,7 +720,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
             __syncthreads();
             uint64_t m[kBatch / kWave];
             batch_hit_mask<kBatch / kWave>(s_rec, s_touch, nb, wave, p.px, p.py, m);
-            if (!want) m[0] = m[1] = m[2] = m[3] = 0;
+            if (!want) {
+#pragma unroll
+                for (int wd = 0; wd < kBatch / kWave; wd++) m[wd] = 0;
+            }
             while (true) {
                 const int e = pop_lowest<kBatch / kWave>(m);
                 if (__builtin_amdgcn_ballot_w64(e >= 0) == 0) break;  // wave-uniform

@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kBinThreads) void tile_ranges_kernel(const uint64_t
 }
 
 // Lower bounds of the per-pixel depths (render.cu:404: interpolate3 of the vertex z with the vertex w
-// as weights) of the rest of every tile list, per batch of kBatch entries.  With positive finite
+// as weights) of the rest of every tile list, per batch of kBoundSpan entries.  With positive finite
 // weights the interpolated depth is a convex combination of the three vertex depths, so it cannot lie
 // below their minimum by more than the rounding of the few operations involved; 32 ulps of the largest
 // |z| are subtracted for that.  An entry with a weight that is not positive and finite bounds nothing
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kBoundThreads) void list_bounds_kernel(const real *
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int tile = blockIdx.x;
     const int start = offsets[tile], n = offsets[tile + 1] - start;
-    const int n_batches = (n + kBatch - 1) / kBatch;
+    const int n_batches = (n + kBoundSpan - 1) / kBoundSpan;
     const real inf = std::numeric_limits<real>::infinity();
     if (threadIdx.x == 0) s_far = n;
     __syncthreads();
@@ -255,8 +255,8 @@ __global__ __launch_bounds__(kBoundThreads) void list_bounds_kernel(const real *
         bool any_far = false;
         int first_far = n;
 #pragma unroll
-        for (int c = kBatch / kWave - 1; c >= 0; c--) {
-            const int p = b * kBatch + c * kWave + lane;
+        for (int c = kBoundSpan / kWave - 1; c >= 0; c--) {
+            const int p = b * kBoundSpan + c * kWave + lane;
             real lb = inf;
             bool far = false;
             if (p < n) {
@@ -269,13 +269,13 @@ __global__ __launch_bounds__(kBoundThreads) void list_bounds_kernel(const real *
             const uint64_t far_lanes = __builtin_amdgcn_ballot_w64(far);
             if (far_lanes) {
                 any_far = true;
-                first_far = b * kBatch + c * kWave + __builtin_ctzll(far_lanes);
+                first_far = b * kBoundSpan + c * kWave + __builtin_ctzll(far_lanes);
             }
             low = (lb < low) ? lb : low;
         }
         low = wave_min(low);
         if (lane == 0) {
-            bounds[batch_bound_index(start, tile, b * kBatch)] = low;
+            bounds[batch_bound_index(start, tile, b * kBoundSpan)] = low;
             if (any_far) atomicMin(&s_far, first_far);
         }
     }
@@ -285,14 +285,14 @@ __global__ __launch_bounds__(kBoundThreads) void list_bounds_kernel(const real *
     real rest = inf;  // bound of everything behind the batches in hand
     for (int hi = n_batches; hi > 0; hi -= kWave) {
         const int b = hi - 1 - lane;  // lane 0 holds the farthest batch
-        real v = (b >= 0) ? bounds[batch_bound_index(start, tile, b * kBatch)] : inf;
+        real v = (b >= 0) ? bounds[batch_bound_index(start, tile, b * kBoundSpan)] : inf;
 #pragma unroll
         for (int d = 1; d < kWave; d <<= 1) {
             const real o = __shfl_up(v, d);
             if (lane >= d) v = (o < v) ? o : v;
         }
         v = (rest < v) ? rest : v;
-        if (b >= 0) bounds[batch_bound_index(start, tile, b * kBatch)] = v;
+        if (b >= 0) bounds[batch_bound_index(start, tile, b * kBoundSpan)] = v;
         rest = __shfl(v, kWave - 1);
     }
     if (lane == 0) far_start[tile] = s_far;
@@ -383,7 +383,7 @@ extern "C" int tg_bary(const real *vertices, int32_t n_vertices, const int32_t *
 
 extern "C" size_t tg_list_bound_words(int64_t n_keys, int n_tiles) {
     if (n_keys < 0 || n_tiles <= 0) return 0;
-    return (size_t)(n_keys / kBatch + n_tiles + 1);
+    return (size_t)(n_keys / kBoundSpan + n_tiles + 1);
 }
 
 extern "C" int tg_list_bounds(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles,

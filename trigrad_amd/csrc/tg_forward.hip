@@ -1,7 +1,7 @@
 // tg_forward.hip -- forward rasterize-and-blend, one workgroup per tile.
 //
 // per_pixel_sort = 0 (tile order): the sorted tile list is staged into LDS in
-//   batches of 256 records; each pixel composites front to back and stops as
+//   batches of 128 records; each pixel composites front to back and stops as
 //   soon as its transmittance falls to the threshold or max_layers fragments
 //   are blended; the workgroup leaves the list when every pixel has stopped.
 // per_pixel_sort = 1: each pixel repeatedly selects its next (up to 32) nearest
@@ -71,7 +71,10 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         // 1. inside tests; a lane keeps its hits as a 256-bit mask
         uint64_t m[kBatch / kWave];
         batch_hit_mask<kBatch / kWave>(s_rec, s_touch, nb, wave, p.px, p.py, m);
-        if (!running) m[0] = m[1] = m[2] = m[3] = 0;
+        if (!running) {
+#pragma unroll
+            for (int wd = 0; wd < kBatch / kWave; wd++) m[wd] = 0;
+        }
         if (masks) {
             // kept for the backward pass, which then has no inside test to repeat
             const int64_t chunk = hit_mask_chunk(start, tile, batch - start);

@@ -13,7 +13,8 @@
 
 namespace tg {
 
-constexpr int kBatch = 256;         // list entries staged per batch
+constexpr int kBatch = 128;         // list entries staged per batch
+constexpr int kBoundSpan = 256;     // list entries per depth bound (tg_list_bounds)
 constexpr int kLayers = 32;         // per-pixel selection batch (render.cu:570, :655)
 constexpr int kMaxTilePixels = 1024;  // tile_w * tile_h limit of the API (wrapper.py:143)
 constexpr int kTileThreads = 256;     // workgroup size limit
@@ -27,7 +28,7 @@ struct RasterArgs {
     const int32_t *sorted_ids;
     const int32_t *offsets;
     const real *bary;
-    const real *batch_bounds;  // per tile and batch of kBatch entries: lower bound of the pixel depths from there on; may be null
+    const real *batch_bounds;  // per tile and kBoundSpan entries: lower bound of the pixel depths from there on; may be null
     const int32_t *far_start;  // per tile: first list position whose entries the bounds do not cover (with batch_bounds)
     int W, H, tw, th;
     real thr;
@@ -139,13 +140,13 @@ __device__ __forceinline__ int64_t hit_mask_head_words() { return (int64_t)gridD
 
 // Batch bounds: word batch_bound_index(start, tile, p) holds, for the tile whose
 // list starts at `start`, a lower bound of the per-pixel depth of every entry at
-// relative position >= p (p a multiple of kBatch) and < far_start[tile].  From
+// relative position >= p (p a multiple of kBoundSpan) and < far_start[tile].  From
 // far_start on the list holds the entries whose clipped polygon was empty (sort
 // key 1e30): they lie at the end of the list whatever their depth, almost never
 // cover a pixel, and are always looked at.  Tiles never share a word;
-// n_keys / kBatch + n_tiles + 1 words hold every list.
+// n_keys / kBoundSpan + n_tiles + 1 words hold every list.
 __device__ __forceinline__ int64_t batch_bound_index(int start, int tile, int relative_position) {
-    return (int64_t)(start / kBatch) + tile + relative_position / kBatch;
+    return (int64_t)(start / kBoundSpan) + tile + relative_position / kBoundSpan;
 }
 
 // Front-to-back compositing state of one pixel (render.cu:564-574).
