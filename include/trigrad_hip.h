@@ -90,6 +90,21 @@ int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t
                           size_t workspace_bytes, uint32_t *status, uint32_t head_stride, uint32_t head_capacity,
                           uint32_t *heads, void *stream);
 
+/* The same scan with nothing to allocate.  It has no counterpart in the
+ * reference: it is for callers that cannot allocate device memory or pass a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  The look-back state lives in a device array inside
+ * the library (64 KiB per GPU, held until the process ends) instead of a
+ * workspace; the call allocates and frees nothing.  n may not exceed
+ * TG_SCAN_NOALLOC_MAX_N = tg_scan_noalloc_max_n() (TG_E_ARG otherwise).  All
+ * calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are safe.  Otherwise as
+ * tg_scan_exclusive_u32, result for result. */
+#define TG_SCAN_NOALLOC_MAX_N (1 << 24)
+int64_t tg_scan_noalloc_max_n(void);
+int tg_scan_exclusive_u32_noalloc(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, uint32_t *status,
+                                  uint32_t head_stride, uint32_t head_capacity, uint32_t *heads, void *stream);
+
 /* Key emission: for triangle i and each tile of its AABB (tile x outer, tile y
  * inner, render.cu:235-236), at position tri_offsets[i] + local:
  *   keys[pos]    = (tile_id << 32) | orderable(depth_key)

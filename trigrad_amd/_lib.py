@@ -34,6 +34,8 @@ SIGNATURES = {
     "tg_bin_count": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _p]),
     "tg_scan_workspace_bytes": (_sz, [_i64]),
     "tg_scan_exclusive_u32": (_i, [_p, _p, _i64, _p, _p, _sz, _p, C.c_uint32, C.c_uint32, _p, _p]),
+    "tg_scan_noalloc_max_n": (_i64, []),
+    "tg_scan_exclusive_u32_noalloc": (_i, [_p, _p, _i64, _p, _p, C.c_uint32, C.c_uint32, _p, _p]),
     "tg_bin_emit": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _i64, _p, C.c_uint32, _p, _p, _p]),
     "tg_sort_workspace_bytes": (_sz, [_i64]),
     "tg_sort_pairs_u64_u32": (_i, [_p, _p, _p, _p, _i64, _i, _p, _sz, _p, C.POINTER(_i), _p]),

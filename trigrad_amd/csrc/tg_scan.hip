@@ -14,6 +14,8 @@
 // at once uses the workgroup ids instead.  The wait is bounded: on
 // expiry the kernel records TG_STATUS_LOOKBACK_TIMEOUT and carries on (with a
 // wrong result) so that every wave still exits.
+#include <mutex>
+
 #include "tg_common.hpp"
 
 namespace tg {
@@ -144,34 +146,31 @@ extern "C" size_t tg_scan_workspace_bytes(int64_t n) {
     return scan_state_offset() + (size_t)tiles * sizeof(uint64_t);
 }
 
-extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
-                                     size_t workspace_bytes, uint32_t *status, uint32_t head_stride, uint32_t head_capacity,
-                                     uint32_t *heads, void *stream) {
+// Argument checks and launches shared by the two entry points; `workspace` holds at least
+// tg_scan_workspace_bytes(n) bytes, 8-byte aligned.
+static int scan_run(const char *fn, const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
+                    uint32_t *status, uint32_t head_stride, uint32_t head_capacity, uint32_t *heads, hipStream_t s) {
     if (n < 0 || !total || !workspace || (n > 0 && (!in || !out))) {
-        set_error("tg_scan_exclusive_u32: null pointer or negative size");
+        set_error("%s: null pointer or negative size", fn);
         return TG_E_ARG;
     }
     if (((uintptr_t)in & 15) || ((uintptr_t)out & 15) || ((uintptr_t)workspace & 7)) {
-        set_error("tg_scan_exclusive_u32: in/out must be 16-byte aligned, workspace 8-byte aligned");
+        set_error("%s: in/out must be 16-byte aligned, workspace 8-byte aligned", fn);
         return TG_E_ARG;
     }
     if (heads && head_stride == 0) {
-        set_error("tg_scan_exclusive_u32: head_stride must be positive when heads is given");
+        set_error("%s: head_stride must be positive when heads is given", fn);
         return TG_E_ARG;
     }
     if (n > (int64_t)kScanTile * 0x7fffffff / 2) {
-        set_error("tg_scan_exclusive_u32: n too large");
+        set_error("%s: n too large", fn);
         return TG_E_ARG;
     }
-    if (workspace_bytes < tg_scan_workspace_bytes(n)) {
-        set_error("tg_scan_exclusive_u32: workspace of %zu bytes, need %zu", workspace_bytes, tg_scan_workspace_bytes(n));
-        return TG_E_WORKSPACE;
-    }
-    hipStream_t s = (hipStream_t)stream;
     const int n_tiles = (int)ceil_div64(n, kScanTile);
     uint32_t *ticket = (uint32_t *)workspace;
     uint64_t *states = (uint64_t *)((char *)workspace + scan_state_offset());
     const int init_blocks = n_tiles > 0 ? ceil_div(n_tiles, 256) : 1;
+    // a kernel, not a memset: the clearing may be recorded into a graph by the caller
     TG_LAUNCH(scan_init_kernel, dim3(init_blocks), dim3(256), 0, s, ticket, states, n_tiles, total, status);
     if (int e = check_launch("scan_init_kernel")) return e;
     if (n_tiles == 0) return 0;
@@ -180,4 +179,64 @@ extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t 
     TG_LAUNCH(scan_lookback_kernel, dim3(n_tiles), dim3(kScanThreads), 0, s, in, out, n, total, ticket, states,
                        n_tiles, status, head_stride, head_capacity, heads);
     return check_launch("scan_lookback_kernel");
+}
+
+extern "C" int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, void *workspace,
+                                     size_t workspace_bytes, uint32_t *status, uint32_t head_stride, uint32_t head_capacity,
+                                     uint32_t *heads, void *stream) {
+    if (n >= 0 && workspace && workspace_bytes < tg_scan_workspace_bytes(n)) {
+        set_error("tg_scan_exclusive_u32: workspace of %zu bytes, need %zu", workspace_bytes, tg_scan_workspace_bytes(n));
+        return TG_E_WORKSPACE;
+    }
+    return scan_run("tg_scan_exclusive_u32", in, out, n, total, workspace, status, head_stride, head_capacity, heads,
+                    (hipStream_t)stream);
+}
+
+// ---- the same scan for callers that cannot allocate ------------------------------------
+// The look-back state (ticket + one word per tile of 2048 elements) lives in a file-scope device array
+// instead of a caller's workspace.  Every GPU the library runs on holds its own copy of the array at its
+// own address, found once per device with hipGetSymbolAddress; host code uses that address only, never the
+// array's name.  All calls on one GPU share the array: calls that overlap there (two streams, two
+// threads) race.  scan_init_kernel clears the part a call uses before the scan reads it.
+constexpr int64_t kStaticScanMaxN = TG_SCAN_NOALLOC_MAX_N;
+constexpr size_t kStaticScanBytes = 64 + (size_t)(kStaticScanMaxN / kScanTile) * sizeof(uint64_t);
+static_assert(kStaticScanMaxN % kScanTile == 0, "whole tiles");
+static __device__ __align__(256) unsigned char scratch[kStaticScanBytes];
+
+static void *static_scan_workspace() {
+    static std::mutex mutex;
+    static void *address[kMaxDevices] = {nullptr};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        set_error("tg_scan_exclusive_u32_noalloc: no current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!address[dev]) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            set_error("tg_scan_exclusive_u32_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        address[dev] = ptr;
+    }
+    return address[dev];
+}
+
+extern "C" int64_t tg_scan_noalloc_max_n(void) { return kStaticScanMaxN; }
+
+extern "C" int tg_scan_exclusive_u32_noalloc(const uint32_t *in, uint32_t *out, int64_t n, uint32_t *total, uint32_t *status,
+                                             uint32_t head_stride, uint32_t head_capacity, uint32_t *heads, void *stream) {
+    if (n > kStaticScanMaxN) {
+        set_error("tg_scan_exclusive_u32_noalloc: n = %lld exceeds the %lld elements the built-in state covers; "
+                  "use tg_scan_exclusive_u32 with a workspace", (long long)n, (long long)kStaticScanMaxN);
+        return TG_E_ARG;
+    }
+    void *workspace = static_scan_workspace();
+    if (!workspace) return TG_E_ARG;
+    return scan_run("tg_scan_exclusive_u32_noalloc", in, out, n, total, workspace, status, head_stride, head_capacity, heads,
+                    (hipStream_t)stream);
 }
