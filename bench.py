@@ -120,11 +120,14 @@ def main():
     sweep_bytes = 24.0 * K
     achieved = sweep_bytes / sweep_avg_s / 1e9
     per_step = {k: v[1] / prof_steps for k, v in prof.items()}
-    bin_sort_kernels = ["bin_count_kernel", "scan_init_kernel", "scan_lookback_kernel", "bin_emit_kernel", "fill_zero_kernel",
-                        "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel", "tile_ranges_kernel"]
+    # binning + sort + ranges: every kernel from the triangles to the sorted tile lists and their offsets
+    sort_kernels = ["fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel",
+                    "segment_sort_small_kernel", "segment_sort_large_kernel"]
+    bin_sort_kernels = ["bin_count_kernel", "scan_init_kernel", "scan_lookback_kernel", "bin_emit_kernel", "bin_init_kernel",
+                        "bin_setup_kernel", "bin_emit_records_kernel", "tile_ranges_kernel"] + sort_kernels
     bin_sort_ms = sum(per_step.get(k, 0.0) for k in bin_sort_kernels)
     bin_sort_bytes = 136.0 * M + 28.0 * K + 24.0 * passes * K + 4.0 * (T + 1)
-    sort_ms = sum(per_step.get(k, 0.0) for k in ("fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel"))
+    sort_ms = sum(per_step.get(k, 0.0) for k in sort_kernels)
 
     out = {
         "metric": "fwd+bwd frames/s (1M tris, 1920x1080)" if args.config == 2 else f"fwd+bwd frames/s (config {args.config})",

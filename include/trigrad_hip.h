@@ -145,6 +145,56 @@ int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, 
  * array that per_tile_lists builds by cumsum (render.cu:292-295). */
 int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int32_t *offsets, void *stream);
 
+/* ---- (2)+(3) for the frame: the tile lists in one call --------------------- */
+
+/* Sorts (tile << 32 | depth bits, triangle) pairs like tg_sort_pairs_u64_u32 on
+ * key bits [0, 32 + bits of n_tiles - 1) and writes the tile ranges like
+ * tg_tile_ranges: same sorted keys, values and offsets, bit for bit.  Replaces
+ * sort_depth_ranges and the offsets of per_tile_lists (render.cu:272-308) for
+ * keys whose high word is a tile number below n_tiles.  It moves the pairs
+ * through memory for the tile bits only (LSD passes of at most 8 bits with
+ * decoupled look-back); the stable passes over the 32 depth bits then run per
+ * tile inside one workgroup, pairs in registers and LDS (a tile list longer
+ * than 8192 entries is sorted by its workgroup through memory instead).
+ * *result_in_alt (host): 0 = sorted data in (keys, values), 1 = in the _alt
+ * pair.  offsets: n_tiles + 1 entries. */
+size_t tg_tile_list_sort_workspace_bytes(int64_t n, int n_tiles);
+int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
+                       int n_tiles, int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status,
+                       int *result_in_alt, void *stream);
+
+/* ---- (1)-(3) as the frame runs them: two calls --------------------------------- */
+
+/* tg_bin_setup = tg_bin_count + tg_scan_exclusive_u32 in one pass over the
+ * triangles (count_per_tile and the cumsum of per_tile_lists, render.cu:90-139,
+ * 290-295): tri_offsets[i] = number of keys of the triangles before i,
+ * total_and_status[0] = K, [1] = TG_STATUS_*.  It also leaves per triangle a
+ * record of TG_RECORD_SCALARS scalars (depth plane of compute_plane,
+ * render.cu:140-152; first tile and rows of the tile rectangle of
+ * touched_tiles, :51-76; the corners) from which tg_build_tile_lists emits the
+ * keys, and in `frame` (tg_bin_setup_workspace_bytes, 256-byte aligned, the
+ * caller's; both calls of a frame get the same one) the state the two calls
+ * share.  heads as in tg_scan_exclusive_u32 with head_stride 256.
+ *
+ * tg_build_tile_lists = tg_bin_emit + tg_sort_tile_lists: emits the K keys from
+ * the records (fill_per_tile_lists_kernel, render.cu:202-270), sorts them and
+ * writes the tile ranges; results as those two calls give them, bit for bit.
+ * While emitting it adds up the digits of the tile passes, so the sort reads
+ * the keys for no histogram.  emit_only != 0: stop after the emission (keys and
+ * values in emission order, as tg_bin_emit leaves them; the double build, whose
+ * depth keys take 64 bits, has this mode only). */
+#define TG_RECORD_SCALARS 12
+size_t tg_bin_setup_workspace_bytes(int32_t n_triangles, int width, int height, int tile_w, int tile_h);
+int tg_bin_setup(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width,
+                 int height, int tile_w, int tile_h, uint32_t *tri_offsets, tg_real *records, uint32_t *total_and_status,
+                 uint32_t head_capacity, uint32_t *heads, void *frame, size_t frame_bytes, void *stream);
+size_t tg_build_tile_lists_workspace_bytes(int64_t n_keys, int n_tiles);
+int tg_build_tile_lists(const tg_real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
+                        uint32_t head_capacity, const uint32_t *heads, void *frame, int width, int height, int tile_w,
+                        int tile_h, uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt,
+                        int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status, int emit_only,
+                        int *result_in_alt, void *stream);
+
 /* ---- bary matrices ---------------------------------------------------------- */
 
 /* Row-major 3x3 cartesian-to-barycentric matrix per triangle, out is (M,3,3).

@@ -94,3 +94,19 @@ def test_product_does_not_reach_into_the_oracle():
 def test_key_bits():
     from trigrad_amd import _C
     assert _C.key_bits(8160) == 45 and _C.key_bits(4096) == 44 and _C.key_bits(256) == 40 and _C.key_bits(1) == 33
+
+
+def test_status_word_check_raises_without_a_gpu():
+    """The check the frame makes of the list kernels' status word, on a host tensor."""
+    import torch
+    from trigrad_amd import _C
+    _C.StatusCheck(torch.zeros((1,), dtype=torch.int32)).verify()
+    bad = _C.StatusCheck(torch.tensor([1], dtype=torch.int32), what="tg_build_tile_lists")
+    with pytest.raises(RuntimeError, match="tg_build_tile_lists: look-back wait timed out"):
+        bad.verify()
+    bad.verify()  # reported once
+    _C._pending_checks.append(_C.StatusCheck(torch.tensor([1], dtype=torch.int32)))
+    with pytest.raises(RuntimeError, match="look-back wait timed out"):
+        _C.verify_finished_frames()
+    _C.verify_finished_frames()
+    assert _C._pending_checks == []

@@ -70,6 +70,15 @@ def test_binning_sort_ranges_full_size(cfg, cuda, oracle):
     ref_offsets, ref_ids, _ = oracle.per_tile_lists(v, idx, W, H)
     np.testing.assert_array_equal(offsets, ref_offsets)
     np.testing.assert_array_equal(sv, ref_ids)
+    # the route the frame takes (one pass for count + scan, emission from records, tile-list sort)
+    setup = _C.bin_setup(d["vertices"], d["indices"], W, H, 16, 16)
+    assert setup["total_and_status"].tolist() == [K, 0]
+    np.testing.assert_array_equal(setup["tri_offsets"].cpu().numpy(), offs.cpu().numpy())
+    fkeys, fids, fstatus, foffsets = _C.build_tile_lists(setup, K)
+    assert int(fstatus.item()) == 0
+    np.testing.assert_array_equal(u64(fkeys), sk)
+    np.testing.assert_array_equal(fids.cpu().numpy(), sv)
+    np.testing.assert_array_equal(foffsets.cpu().numpy(), ref_offsets)
     # properties that need no oracle
     assert (np.diff(sk.astype(np.uint64)) >= 0).all() if K > 1 else True
     assert offsets[0] == 0 and offsets[-1] == K and (np.diff(offsets) >= 0).all()

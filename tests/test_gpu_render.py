@@ -42,14 +42,14 @@ def _forward_both(scene, tw, th, mode, cuda, oracle, thr=1 / 256):
     ml = mode["max_layers"] if mode["max_layers"] > 0 else M + 1
     want = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H, tw, th, thr,
                          mode["per_pixel_sort"], ml)
-    got = _C.render_forward(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, thr, True,
+    got = _C._forward_full(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, thr, True,
                             mode["per_pixel_sort"], ml)
     return d, want, got, ml
 
 
 def _check_forward(name, want, got):
     image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status, fragments, hit_masks) = got
-    assert int(status.item()) == 0
+    status.verify()
     np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
     np.testing.assert_array_equal(sorted_ids.cpu().numpy(), want["sorted_ids"])
     img = image.cpu().numpy()
@@ -265,7 +265,7 @@ def test_selection_early_stop_changes_nothing(name, mode, cuda, monkeypatch):
     outs = []
     for threshold in (1 << 30, 0):  # never / always
         monkeypatch.setattr(_C, "EARLY_STOP_MIN_AVG_LIST", threshold)
-        outs.append(_C.render_forward(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, 1 / 256, True, True, ml))
+        outs.append(_C._forward_full(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, 1 / 256, True, True, ml))
     for a, b in zip(outs[0][:7], outs[1][:7]):
         assert torch.equal(a.view(torch.int32) if a.is_floating_point() else a, b.view(torch.int32) if b.is_floating_point() else b)
     ra, rb = outs[0][8], outs[1][8]
@@ -353,3 +353,109 @@ def test_argument_errors(cuda):
         trigrad_amd.render(v, i, c[:-1], o)
     with pytest.raises(TypeError, match="opacities must be of type torch.float32"):
         trigrad_amd.render(v, i, c, o.double())
+
+
+class _ReferenceShapedRenderer:
+    """The call pattern of the reference's autograd Function (src/trigrad/wrapper.py:56-70, 87-98): twelve arguments
+    into render_forward, eight results out, exactly eleven tensors saved, twenty arguments into render_backward."""
+
+    @staticmethod
+    def make(drop_private_state):
+        import torch
+        from trigrad_amd import _C
+
+        class Fn(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, vertices, indices, colors, opacities, width, height, tw, th, thr, record_timing, pps, max_layers):
+                ctx.args = (width, height, tw, th, thr, pps, max_layers)
+                image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings = _C.render_forward(
+                    vertices, indices, colors, opacities, width, height, tw, th, thr, not record_timing, pps, max_layers)
+                if drop_private_state:
+                    del ends._tg_resume
+                ctx.save_for_backward(vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, image, depthmap,
+                                      final_weights, ends)
+                return image, depthmap
+
+            @staticmethod
+            def backward(ctx, grad_image, grad_depthmap):
+                gv, gc, go = _C.render_backward(grad_image, grad_depthmap, *ctx.saved_tensors, *ctx.args)
+                return (gv, None, gc, go) + (None,) * 8
+
+        return Fn
+
+
+@pytest.mark.parametrize("drop_private_state", [False, True])
+@pytest.mark.parametrize("mode", ["A_default", "B_unlimited", "B_3_layers", "A_40_layers"])
+def test_native_surface_as_the_reference_wrapper_calls_it(mode, drop_private_state, cuda, oracle):
+    """_C.render_forward / _C.render_backward with the reference's argument lists and nothing else carried over:
+    with the private state that travels on `ends`, and after a caller lost it (it is then computed again)."""
+    import torch
+    from trigrad_amd import scenes as S
+    scene = S.random_soup(700, 150, 110, seed=21, sigma_px=11.0, varying_w=True)
+    m = MODES[mode]
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    ml = m["max_layers"] if m["max_layers"] > 0 else scene["indices"].shape[0] + 1
+    v = d["vertices"].clone().requires_grad_()
+    c = d["colors"].clone().requires_grad_()
+    o = d["opacities"].clone().requires_grad_()
+    Fn = _ReferenceShapedRenderer.make(drop_private_state)
+    image, depthmap = Fn.apply(v, d["indices"], c, o, W, H, 16, 16, 1 / 256, False, m["per_pixel_sort"], ml)
+    rng = np.random.default_rng(5)
+    gi = rng.standard_normal((H, W, 4)).astype(np.float32)
+    gd = rng.standard_normal((H, W)).astype(np.float32)
+    want = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H, 16, 16, 1 / 256,
+                         m["per_pixel_sort"], ml)
+    assert int((image.detach().cpu().numpy().view(np.uint32) != want["image"].view(np.uint32)).sum()) == 0
+    finite = np.isfinite(want["depthmap"])
+    gd = np.where(finite, gd, 0).astype(np.float32)
+    torch.autograd.backward([image, depthmap], [torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda)])
+    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                        W, H, 16, 16, m["per_pixel_sort"], ml)
+    for label, got, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
+        assert_close(f"{mode}: {label}", got.cpu().numpy(), w, 1e-4, 1e-6 + 2e-6 * float(np.abs(w).max()))
+
+
+def test_expired_wait_is_reported_on_every_path(cuda):
+    """A non-zero status word of the list kernels (a bounded look-back wait expired: the lists are invalid) raises in
+    the backward pass and at the start of the next frame, not only when timings are recorded.  No wait is provoked:
+    the status word is forged."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import _C, scenes as S
+    d = to_device(S.config(0), cuda)
+    args = (d["vertices"], d["indices"], d["colors"], d["opacities"], 256, 256, 16, 16, 1 / 256)
+    *results, resume = _C._forward_full(*args, True, False, 2000)
+    image, depthmap, weights, sorted_ids, offsets, bary, ends = results[:7]
+    bad = _C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda))
+    gi = torch.ones_like(image)
+    with pytest.raises(RuntimeError, match="look-back wait timed out"):
+        _C.render_backward(gi, None, *args[:4], sorted_ids, offsets, bary, image, depthmap, weights, ends, *args[4:], False, 2000,
+                           resume=(resume[0], resume[1], bad, resume[3], resume[4]))
+    # the same through the public entry point: the next frame refuses to start
+    _C._pending_checks.append(_C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda)))
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="look-back wait timed out"):
+        trigrad_amd.render(*args[:6])
+    assert not _C._pending_checks or all(not c.checked for c in _C._pending_checks)
+    trigrad_amd.render(*args[:6])  # reported once; later frames run
+    # and a healthy frame's word is zero
+    resume[2].verify()
+
+
+@pytest.mark.parametrize("mode", ["A_default", "B_unlimited"])
+def test_scene_without_a_single_key(mode, cuda):
+    """M >= 1 but K = 0 (every triangle degenerate): transparent image, infinite depth, zero gradients."""
+    import torch
+    import trigrad_amd
+    m = MODES[mode]
+    v = torch.tensor([[0.1, 0.1, 0.5, 2.0]] * 3 + [[float("nan"), 0.0, 0.5, 1.0], [0.2, 0.3, 0.5, 1.0], [0.4, 0.1, 0.5, 1.0]],
+                     dtype=torch.float32, device=cuda).requires_grad_()
+    idx = torch.tensor([[0, 1, 2], [3, 4, 5], [0, 0, 4]], dtype=torch.int32, device=cuda)
+    c = torch.rand((6, 3), device=cuda).requires_grad_()
+    o = torch.rand((6,), device=cuda).requires_grad_()
+    image, depthmap = trigrad_amd.render(v, idx, c, o, 70, 50, 16, 16, 1 / 256, False, m["per_pixel_sort"], m["max_layers"])
+    assert float(image[..., :3].abs().max()) == 0.0 and float(image[..., 3].min()) == 1.0 and torch.isinf(depthmap).all()
+    (image.sum() + torch.where(torch.isinf(depthmap), torch.zeros_like(depthmap), depthmap).sum()).backward()
+    for g in (v.grad, c.grad, o.grad):
+        assert float(g.abs().max()) == 0.0

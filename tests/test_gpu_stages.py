@@ -107,6 +107,21 @@ def test_binning_sort_ranges_bit_exact(name, cuda, oracle):
     np.testing.assert_array_equal(svals.cpu().numpy(), ref_ids)
     np.testing.assert_array_equal(np.diff(ref_offsets), tile_counts)
 
+    # the frame's route: count + scan in one pass, emission from the triangles' records, tile bits sorted
+    # through memory and depth bits per tile in LDS
+    for with_heads in (True, False):
+        setup = _C.bin_setup(d["vertices"], d["indices"], W, H, tw, th, with_heads=with_heads)
+        assert setup["total_and_status"].tolist() == [K, 0]
+        np.testing.assert_array_equal(setup["tri_offsets"].cpu().numpy(), np.cumsum(tri_counts) - tri_counts)
+        ekeys, epayload, estatus, _ = _C.build_tile_lists(setup, K, emit_only=True)
+        np.testing.assert_array_equal(u64(ekeys), em["keys64"])
+        np.testing.assert_array_equal(epayload.cpu().numpy(), em["tri"])
+        fkeys, fids, fstatus, foffsets = _C.build_tile_lists(setup, K)
+        assert int(fstatus.item()) == 0
+        np.testing.assert_array_equal(u64(fkeys), want_keys)
+        np.testing.assert_array_equal(fids.cpu().numpy(), want_vals)
+        np.testing.assert_array_equal(foffsets.cpu().numpy(), ref_offsets)
+
     got_bary = _C.cartesian_to_bary(d["vertices"], d["indices"]).cpu().numpy()
     want_bary = oracle.bary(v, idx)
     np.testing.assert_array_equal(got_bary.view(np.uint32), want_bary.view(np.uint32))
@@ -207,3 +222,65 @@ def test_out_of_range_indices_are_skipped(cuda):
     d = to_device(s, cuda)
     counts = _C.bin_count(d["vertices"], torch.from_numpy(idx).to(cuda), 64, 64, 16, 16).cpu().numpy()
     assert counts[4] == 0 and counts[7] == 0 and (np.delete(counts, [4, 7]) > 0).all()
+
+
+def _tile_list_case(n, n_tiles, rng, depth_pool=None, skew=None):
+    """Random (tile << 32 | depth bits) keys; skew: a share of the keys goes to one tile (a long list)."""
+    tiles = rng.integers(0, n_tiles, size=n, dtype=np.uint64)
+    if skew:
+        tiles[rng.random(n) < skew] = np.uint64(n_tiles // 2)
+    if depth_pool:
+        depth = rng.integers(0, 1 << 32, size=depth_pool, dtype=np.uint64)[rng.integers(0, depth_pool, size=n)]
+    else:
+        depth = rng.integers(0, 1 << 32, size=n, dtype=np.uint64)
+    return (tiles << np.uint64(32)) | depth
+
+
+@pytest.mark.parametrize("n,n_tiles,depth_pool,skew", [
+    (1, 1, None, None), (2, 7, None, None), (300, 1, None, None), (5000, 256, None, None), (70_000, 300, 3, None),
+    (200_000, 8160, None, None), (200_000, 8160, 50, 0.02),       # one list of about 4000 entries among short ones
+    (300_000, 97, None, None),                                    # every list between 2048 and 4096 entries
+    (400_000, 64, None, None), (700_000, 128, 1000, None),        # 6250 and 5500 entries a list
+    (60_000, 3, None, None), (50_000, 5, 2, 0.9),                 # lists longer than the LDS holds; few distinct depths
+    (3_000_000, 8160, None, None), (5_000_017, 1024, None, 0.001),  # more sort tiles than fit the device at once
+])
+def test_sort_tile_lists_matches_stable_sort(n, n_tiles, depth_pool, skew, cuda):
+    """The tile-list sort (tile bits through memory, depth bits per tile in LDS) against numpy's stable argsort
+    of the whole key, and its ranges against searchsorted."""
+    import torch
+    from trigrad_amd import _C
+    rng = np.random.default_rng(n + n_tiles)
+    keys = _tile_list_case(n, n_tiles, rng, depth_pool, skew)
+    vals = np.arange(n, dtype=np.int32)
+    order = np.argsort(keys, kind="stable")
+    k = torch.from_numpy(keys.view(np.int64).copy()).to(cuda)
+    v = torch.from_numpy(vals.copy()).to(cuda)
+    sk, sv, status, offsets = _C.sort_tile_lists(k, v, n_tiles)
+    assert int(status.item()) == 0
+    np.testing.assert_array_equal(u64(sk), keys[order])
+    np.testing.assert_array_equal(sv.cpu().numpy(), vals[order])
+    np.testing.assert_array_equal(offsets.cpu().numpy(), np.searchsorted(keys[order] >> np.uint64(32), np.arange(n_tiles + 1)))
+
+
+def test_sort_tile_lists_uniform_digits_and_empty(cuda):
+    """Depth words that differ in one byte only (three of the four passes are left out), equal keys, no keys."""
+    import torch
+    from trigrad_amd import _C
+    rng = np.random.default_rng(3)
+    for byte in range(4):
+        n, T = 40_000, 50
+        depth = np.uint64(0x3A5C77E1) & ~np.uint64(0xFF << (8 * byte)) | (rng.integers(0, 256, size=n, dtype=np.uint64) << np.uint64(8 * byte))
+        keys = (rng.integers(0, T, size=n, dtype=np.uint64) << np.uint64(32)) | depth
+        order = np.argsort(keys, kind="stable")
+        sk, sv, status, offsets = _C.sort_tile_lists(torch.from_numpy(keys.view(np.int64).copy()).to(cuda),
+                                                     torch.arange(n, dtype=torch.int32, device=cuda), T)
+        np.testing.assert_array_equal(u64(sk), keys[order])
+        np.testing.assert_array_equal(sv.cpu().numpy(), order.astype(np.int32))
+    keys = np.full(9000, (np.uint64(3) << np.uint64(32)) | np.uint64(77), dtype=np.uint64)
+    sk, sv, status, offsets = _C.sort_tile_lists(torch.from_numpy(keys.view(np.int64).copy()).to(cuda),
+                                                 torch.arange(9000, dtype=torch.int32, device=cuda), 6)
+    np.testing.assert_array_equal(sv.cpu().numpy(), np.arange(9000, dtype=np.int32))
+    assert offsets.tolist() == [0, 0, 0, 0, 9000, 9000, 9000]
+    sk, sv, status, offsets = _C.sort_tile_lists(torch.empty((0,), dtype=torch.int64, device=cuda),
+                                                 torch.empty((0,), dtype=torch.int32, device=cuda), 300)
+    assert sk.numel() == 0 and int(status.item()) == 0 and offsets.tolist() == [0] * 301

@@ -176,6 +176,87 @@ def tile_ranges(sorted_keys, n_tiles):
     return offsets
 
 
+def sort_tile_lists(keys, values, n_tiles):
+    """(tile << 32 | depth bits, triangle) pairs -> (sorted_keys, sorted_values, status (1,) int32, offsets (T+1,) int32).
+
+    Same result as sort_pairs on key_bits(n_tiles) followed by tile_ranges; the passes over the depth bits run
+    per tile inside a workgroup.  The inputs are used as scratch."""
+    _need_cuda(keys, values)
+    lib = _lib.load()
+    n = keys.numel()
+    dev = keys.device
+    keys_alt = torch.empty_like(keys)
+    values_alt = torch.empty_like(values)
+    status = torch.empty((1,), dtype=torch.int32, device=dev)
+    offsets = torch.empty((n_tiles + 1,), dtype=torch.int32, device=dev)
+    ws_bytes = int(lib.tg_tile_list_sort_workspace_bytes(n, n_tiles))
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    in_alt = C.c_int(0)
+    with _on_device(dev):
+        _lib.check(lib.tg_sort_tile_lists(_ptr(keys), _ptr(values), _ptr(keys_alt), _ptr(values_alt), n, n_tiles, _ptr(offsets),
+                                          _ptr(ws), ws_bytes, _ptr(status), C.byref(in_alt), _stream(keys)), "tg_sort_tile_lists")
+    if in_alt.value:
+        return keys_alt, values_alt, status, offsets
+    return keys, values, status, offsets
+
+
+RECORD_SCALARS = 12  # TG_RECORD_SCALARS of the C header
+
+
+def bin_setup(vertices, indices, width, height, tile_width, tile_height, with_heads=True):
+    """Counts, scans and prepares the emission in one pass over the triangles.
+
+    -> dict(tri_offsets (M,) int32, records (M, 12), total_and_status (2,) int32, heads, frame, geometry)"""
+    _need_cuda(vertices, indices)
+    bits = _bits(vertices)
+    lib = _lib.load(bits)
+    dev = vertices.device
+    M = indices.shape[0]
+    tri_offsets = torch.empty((M,), dtype=torch.int32, device=dev)
+    records = torch.empty((M, RECORD_SCALARS), dtype=vertices.dtype, device=dev)
+    pair = torch.empty((2,), dtype=torch.int32, device=dev)
+    heads = owner_heads_for(M, dev) if with_heads else None
+    frame_bytes = int(lib.tg_bin_setup_workspace_bytes(M, width, height, tile_width, tile_height))
+    frame = torch.empty((frame_bytes,), dtype=torch.uint8, device=dev)
+    with _on_device(dev):
+        _lib.check(lib.tg_bin_setup(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
+                                    _ptr(tri_offsets), _ptr(records), _ptr(pair), 0 if heads is None else heads.numel(), _ptr(heads),
+                                    _ptr(frame), frame_bytes, _stream(vertices)), "tg_bin_setup", bits)
+    return dict(tri_offsets=tri_offsets, records=records, total_and_status=pair, heads=heads, frame=frame,
+                geometry=(width, height, tile_width, tile_height), bits=bits)
+
+
+def build_tile_lists(setup, n_keys, emit_only=False):
+    """bin_setup's result + K -> (sorted_keys, sorted_ids, status (1,) int32, offsets (T+1,) int32);
+    emit_only: (keys, ids, status, None) in emission order (float64: 2K keys, depth keys then tile ids)."""
+    bits = setup["bits"]
+    lib = _lib.load(bits)
+    records, tri_offsets, heads, frame = setup["records"], setup["tri_offsets"], setup["heads"], setup["frame"]
+    width, height, tile_width, tile_height = setup["geometry"]
+    dev = records.device
+    T = num_tiles(width, height, tile_width, tile_height)
+    keys = torch.empty((n_keys * (2 if bits == 64 else 1),), dtype=torch.int64, device=dev)
+    values = torch.empty((n_keys,), dtype=torch.int32, device=dev)
+    status = torch.empty((1,), dtype=torch.int32, device=dev)
+    keys_alt = values_alt = offsets = ws = None
+    ws_bytes = 0
+    if not emit_only:
+        keys_alt, values_alt = torch.empty_like(keys), torch.empty_like(values)
+        offsets = torch.empty((T + 1,), dtype=torch.int32, device=dev)
+        ws_bytes = int(lib.tg_build_tile_lists_workspace_bytes(n_keys, T))
+        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    in_alt = C.c_int(0)
+    with _on_device(dev):
+        _lib.check(lib.tg_build_tile_lists(_ptr(records), _ptr(tri_offsets), tri_offsets.numel(), n_keys,
+                                           0 if heads is None else heads.numel(), _ptr(heads), _ptr(frame), width, height,
+                                           tile_width, tile_height, _ptr(keys), _ptr(values), _ptr(keys_alt), _ptr(values_alt),
+                                           _ptr(offsets), _ptr(ws), ws_bytes, _ptr(status), int(bool(emit_only)), C.byref(in_alt),
+                                           _stream(records)), "tg_build_tile_lists", bits)
+    if in_alt.value:
+        return keys_alt, values_alt, status, offsets
+    return keys, values, status, offsets
+
+
 def cartesian_to_bary(vertices, indices):
     """(M,3,3) cartesian-to-barycentric matrices (reference _C.cartesian_to_bary, render.cu:697-711)."""
     _need_cuda(vertices, indices)
@@ -257,16 +338,64 @@ class _StageTimer:
         return {name: evs[k].elapsed_time(evs[k + 1]) / 1000.0 for k, (name, _) in enumerate(self.marks)}
 
 
-def render_forward(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
-                   early_stopping_threshold, disable_timing, per_pixel_sort, max_layers):
-    """Reference _C.render_forward (render.cu:713-763).
+class StatusCheck:
+    """The status word of the kernels that wait on other workgroups (TG_STATUS_*), on its way to the host.
 
-    -> (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume)
-    `resume` = (last, last_depth, status, fragments, hit_masks): what the backward
-    pass needs for its reverse traversal (fragments / hit_masks are None unless the
-    blend order / the hit masks were saved), plus the sort's status word.
-    """
+    The word is copied to pinned host memory behind the kernels that write it, without a wait; `verify`
+    waits for that copy (long done when the backward pass or the next frame asks) and raises RuntimeError
+    if a bounded wait expired, because the lists and everything rendered from them are then invalid."""
+
+    def __init__(self, status, what="tg_build_tile_lists"):
+        self.what = what
+        self.checked = False
+        if status.device.type == "cuda":
+            self.host = torch.empty((status.numel(),), dtype=torch.int32, pin_memory=True)
+            self.host.copy_(status, non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record(torch.cuda.current_stream(status.device))
+        else:
+            self.host = status.clone()
+            self.event = None
+
+    def ready(self):
+        return self.event is None or self.event.query()
+
+    def verify(self):
+        if self.checked:
+            return
+        if self.event is not None:
+            self.event.synchronize()
+        self.checked = True
+        if int(self.host.max()) != 0:
+            raise RuntimeError(f"{self.what}: look-back wait timed out (status {self.host.tolist()}); the frame is invalid")
+
+
+_pending_checks = []  # status words of earlier frames that nobody has looked at yet
+
+
+def verify_finished_frames():
+    """Raises for any earlier frame whose status word has arrived and reports a timeout; never waits."""
+    still = []
+    try:
+        while _pending_checks:
+            check = _pending_checks.pop(0)
+            if check.checked:
+                continue
+            if check.ready():
+                check.verify()
+            else:
+                still.append(check)
+    finally:
+        _pending_checks[:0] = still
+
+
+def _forward_full(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                  early_stopping_threshold, disable_timing, per_pixel_sort, max_layers):
+    """render_forward's eight results plus `resume` = (last, last_depth, status_check, fragments, hit_masks):
+    what the backward pass needs for its reverse traversal (fragments / hit_masks are None unless the blend
+    order / the hit masks were saved) and the status word of the list kernels on its way to the host."""
     _need_cuda(vertices, indices, colors, opacities)
+    verify_finished_frames()
     bits = _bits(vertices)
     lib = _lib.load(bits)
     real = vertices.dtype
@@ -289,28 +418,35 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
 
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
-        counts = bin_count(vertices, indices, width, height, tile_width, tile_height)
-        heads = owner_heads_for(indices.shape[0], dev)
-        tri_offsets, total, status = scan_exclusive(counts, out=counts, heads=heads)
+        setup = bin_setup(vertices, indices, width, height, tile_width, tile_height)
         bary_transforms = None
         if disable_timing:
             # K travels to pinned host memory while the device already computes the bary matrices, which do
             # not depend on it; the host waits for the copy only (with stage timings the reference's order is kept)
             host = torch.empty((2,), dtype=torch.int32, pin_memory=True)
-            host.copy_(total._base, non_blocking=True)
+            host.copy_(setup["total_and_status"], non_blocking=True)
             arrived = torch.cuda.Event()
             arrived.record()
             bary_transforms = cartesian_to_bary(vertices, indices)
             arrived.synchronize()
         else:
-            host = total._base.cpu()
+            host = setup["total_and_status"].cpu()
         K, st = host.tolist()  # one conversion: the device waits for the launches that follow
         if st != 0:
-            raise RuntimeError("tg_scan_exclusive_u32: look-back wait timed out")
-        keys, payload = bin_emit(vertices, indices, tri_offsets, K, width, height, tile_width, tile_height, heads)
-
-        timer.start("sorting")
-        keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
+            raise RuntimeError("tg_bin_setup: look-back wait timed out")
+        if bits == 32 and disable_timing:
+            keys, sorted_ids, sort_status, offsets = build_tile_lists(setup, K)
+        else:
+            # the stages apart, so that their times are the reference's (render.cu:733-745); the double build's
+            # depth keys take 64 bits and are sorted in two rounds
+            keys, payload, _, _ = build_tile_lists(setup, K, emit_only=True)
+            timer.start("sorting")
+            if bits == 32:
+                keys, sorted_ids, sort_status, offsets = sort_tile_lists(keys, payload, T)
+            else:
+                keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
+        status_check = StatusCheck(sort_status)
+        _pending_checks.append(status_check)
 
         timer.start("bary_transforms")
         if bary_transforms is None:
@@ -336,29 +472,82 @@ def render_forward(vertices, indices, colors, opacities, width, height, tile_wid
             _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
             _ptr(hit_masks), _ptr(batch_bounds), _ptr(far_start), _stream(vertices)), "tg_render_forward", bits)
         timings = timer.stop()
+        if not disable_timing:
+            status_check.verify()  # the timer has waited for the stream anyway
     return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
-            (last, last_depth, sort_status, fragments, hit_masks))
+            (last, last_depth, status_check, fragments, hit_masks))
+
+
+def render_forward(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                   early_stopping_threshold, disable_timing, per_pixel_sort, max_layers):
+    """Reference _C.render_forward (render.h:22-36, render.cu:713-763), same arguments, same eight results:
+
+    -> (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings)
+
+    What this build's backward pass wants beyond them travels as an attribute of `ends` (render_backward
+    looks for it there and does without if it is gone)."""
+    *results, resume = _forward_full(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                                     early_stopping_threshold, disable_timing, per_pixel_sort, max_layers)
+    results[6]._tg_resume = resume
+    return tuple(results)
+
+
+def _resume_by_forward(vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, width, height, tile_width,
+                       tile_height, early_stopping_threshold, per_pixel_sort, max_layers):
+    """What the forward kernel hands to the backward pass, computed again from the saved lists: the forward
+    kernel runs once more into scratch outputs (a caller that kept only the reference's saved tensors)."""
+    bits = _bits(vertices)
+    lib = _lib.load(bits)
+    real, dev = vertices.dtype, vertices.device
+    image = torch.empty((height, width, 4), dtype=real, device=dev)
+    plane = [torch.empty((height, width), dtype=real, device=dev) for _ in range(2)]
+    ends = torch.empty((height, width), dtype=torch.int32, device=dev)
+    last = torch.empty((height, width), dtype=torch.int32, device=dev)
+    last_depth = torch.empty((height, width), dtype=real, device=dev) if per_pixel_sort else None
+    save_order = bool(per_pixel_sort) and SAVE_BLEND_ORDER and 0 < int(max_layers) <= MAX_SAVED_LAYERS
+    fragments = torch.empty((int(max_layers), height, width), dtype=torch.int32, device=dev) if save_order else None
+    hit_masks = None
+    if not per_pixel_sort and SAVE_HIT_MASKS:
+        words = int(lib.tg_hit_mask_words(sorted_ids.numel(), width, height, tile_width, tile_height))
+        hit_masks = torch.empty((words,), dtype=torch.int64, device=dev)
+    _lib.check(lib.tg_render_forward(
+        _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
+        width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
+        _ptr(image), _ptr(plane[0]), _ptr(plane[1]), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
+        _ptr(hit_masks), None, None, _stream(vertices)), "tg_render_forward", bits)
+    return last, last_depth, None, fragments, hit_masks
 
 
 def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms,
                     image, depthmap, final_weights, ends, width, height, tile_width, tile_height, early_stopping_threshold,
                     per_pixel_sort, max_layers, resume=None, grad_strides=None):
-    """Reference _C.render_backward (render.cu:765-804) -> (grad_vertices, grad_colors, grad_opacities).
+    """Reference _C.render_backward (render.h:6-20, render.cu:765-804), same twenty arguments
+    -> (grad_vertices, grad_colors, grad_opacities).
 
-    grad_depthmap may be None (no gradient reached the depth map).  grad_strides (scalars per vertex in the
-    three arrays the kernel accumulates into) defaults to dense arrays in tile order and to one (V,8) block
-    with per_pixel_sort; the returned tensors are dense either way."""
-    if resume is None:
-        raise ValueError("render_backward needs the `resume` tuple returned by render_forward")
-    last, last_depth, sort_status, fragments, hit_masks = resume
+    resume: what _forward_full returned next to the reference's results; without it (the reference's wrapper
+    saves eleven tensors and nothing else) it is taken from `ends` if render_forward's attribute is still
+    there, else computed again.  grad_depthmap may be None (no gradient reached the depth map).  grad_strides
+    (scalars per vertex in the three arrays the kernel accumulates into) defaults to dense arrays in tile order
+    and to one (V,8) block with per_pixel_sort; the returned tensors are dense either way."""
     _need_cuda(grad_output, vertices)
+    if max_layers <= 0:
+        max_layers = indices.shape[0] + 1
     bits = _bits(vertices)
     lib = _lib.load(bits)
     dev = vertices.device
     with _on_device(dev):
         tensors = [None if t is None else t.contiguous()
                    for t in (grad_output, grad_depthmap, vertices, indices, colors, opacities, sorted_ids, offsets,
-                             bary_transforms, image, depthmap, final_weights, ends, last)]
+                             bary_transforms, image, depthmap, final_weights, ends)]
+        if resume is None:
+            resume = getattr(ends, "_tg_resume", None)
+        if resume is None:
+            resume = _resume_by_forward(*tensors[2:9], width, height, tile_width, tile_height, early_stopping_threshold,
+                                        per_pixel_sort, max_layers)
+        last, last_depth, status_check, fragments, hit_masks = resume
+        if status_check is not None:
+            status_check.verify()
+        tensors.append(last.contiguous())
         # one zero fill for the three gradients.  Tile order: (V,4) | (V,3) | (V,) views of one block.  Per-pixel
         # order issues five times as many atomics; there the eight gradients of a vertex share a 32-byte
         # sector of a (V,8) block while the kernel runs, and the three arrays are copied out afterwards.

@@ -40,6 +40,13 @@ SIGNATURES = {
     "tg_sort_workspace_bytes": (_sz, [_i64]),
     "tg_sort_pairs_u64_u32": (_i, [_p, _p, _p, _p, _i64, _i, _p, _sz, _p, C.POINTER(_i), _p]),
     "tg_tile_ranges": (_i, [_p, _i64, _i, _p, _p]),
+    "tg_tile_list_sort_workspace_bytes": (_sz, [_i64, _i]),
+    "tg_sort_tile_lists": (_i, [_p, _p, _p, _p, _i64, _i, _p, _p, _sz, _p, C.POINTER(_i), _p]),
+    "tg_bin_setup_workspace_bytes": (_sz, [_i32, _i, _i, _i, _i]),
+    "tg_bin_setup": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _p, _p, C.c_uint32, _p, _p, _sz, _p]),
+    "tg_build_tile_lists_workspace_bytes": (_sz, [_i64, _i]),
+    "tg_build_tile_lists": (_i, [_p, _p, _i32, _i64, C.c_uint32, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p, _i,
+                                C.POINTER(_i), _p]),
     "tg_bary": (_i, [_p, _i32, _p, _i32, _p, _p]),
     "tg_list_bound_words": (_sz, [_i64, _i]),
     "tg_list_bounds": (_i, [_p, _i32, _p, _i32, _p, _p, _p, _i, _p, _p, _p, _p]),

@@ -1,6 +1,6 @@
-// tg_binning.hip -- tile binning (count, key emission), tile ranges and bary matrices.
+// tg_binning.hip -- tile binning (count, key emission) and bary matrices.
 //
-// count, ranges and bary are HBM-bound streaming kernels; emit is bound by the
+// count and bary are HBM-bound streaming kernels; emit is bound by the
 // clipping arithmetic it does per key:
 //   count   reads 12 B indices + 3 x 16 B vertex gathers, writes 4 B per triangle
 //   emit    one thread per KEY (not per triangle), so a triangle that covers
@@ -8,9 +8,10 @@
 //           triangle again (L2 hits for neighbouring keys), clips it to the
 //           tile (polygon in LDS), writes 8 B key + 4 B payload per key,
 //           coalesced
-//   ranges  reads 8 B per sorted key, writes 4 B per tile
 //   bary    reads 60 B, writes 36 B per triangle
 #include "tg_raster.hpp"
+#include "tg_scan.hpp"
+#include "tg_sort_plan.hpp"
 
 namespace tg {
 
@@ -194,13 +195,235 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
     payload[k] = (uint32_t)t;
 }
 
-__global__ __launch_bounds__(kBinThreads) void tile_ranges_kernel(const uint64_t *__restrict__ sorted_keys, int64_t n_keys,
-                                                                  int n_tiles, int32_t *__restrict__ offsets) {
-    const int64_t i = (int64_t)blockIdx.x * kBinThreads + threadIdx.x;
-    if (i > n_keys) return;
-    const int cur = (i < n_keys) ? (int)(sorted_keys[i] >> 32) : n_tiles;
-    const int prev = (i > 0) ? (int)(sorted_keys[i - 1] >> 32) : -1;
-    for (int t = prev + 1; t <= cur && t <= n_tiles; t++) offsets[t] = (int32_t)i;
+// ---- the frame's binning in two launches ---------------------------------------------------------------
+//
+// bin_setup_kernel counts and scans in one pass over the triangles (the tile's count total goes through the
+// same decoupled look-back as the plain scan) and leaves, per triangle, a record of what the emission needs
+// for each of its keys: the depth plane, the first tile and the rows of the tile rectangle, the three
+// corners.  bin_emit_records_kernel then reads one record per key instead of the triangle's indices and
+// vertices, and does per key only what depends on the tile: the clip and the minimum.
+//
+// Frame state (caller's memory, tg_bin_setup_workspace_bytes): scan ticket, the sort's tickets and queue
+// length, the digit totals of the tile passes, the NDC edges of the tile columns and rows, the scan's state
+// words.  bin_init_kernel clears it and fills in the edges.
+constexpr int kRecordReals = TG_RECORD_SCALARS;  // A B C x0 | ax ay bx by | cx cy y0 ny
+static_assert(kRecordReals == 12, "three real4 per triangle");
+constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets; kQueueCountWord: queued segments
+constexpr int kStateTotalsWords = (kMaxPasses / 2) * kRadix;
+static_assert(kQueueCountWord < kStateTicketWords, "the queue length lives in the ticket block");
+
+struct FrameState {
+    uint32_t *tickets;
+    uint32_t *totals;
+    real *edges;       // tiles_x + 1 column edges, then tiles_y + 1 row edges
+    uint64_t *states;  // one per kScanTile triangles
+    size_t bytes;
+};
+
+static FrameState frame_state(void *base, int64_t n_triangles, int tiles_x, int tiles_y) {
+    FrameState f;
+    char *p = (char *)base;
+    size_t o = 0;
+    f.tickets = (uint32_t *)(p + o); o += kStateTicketWords * 4;
+    f.totals = (uint32_t *)(p + o);  o += kStateTotalsWords * 4;
+    f.states = (uint64_t *)(p + o);  o += (size_t)(ceil_div64(n_triangles, kScanTile) + 1) * 8;
+    f.edges = (real *)(p + o);       o += (size_t)(tiles_x + tiles_y + 2) * sizeof(real);
+    f.bytes = (o + 255) & ~(size_t)255;
+    return f;
+}
+
+__global__ __launch_bounds__(1024) void bin_init_kernel(uint32_t *zero, size_t zero_words, real *edges, int W, int H, int tw, int th,
+                                                        int tiles_x, int tiles_y, uint32_t *total_and_status) {
+    for (size_t i = threadIdx.x; i < zero_words; i += blockDim.x) zero[i] = 0;
+    // render.cu:243-246: the edges of tile column tx are entries tx and tx + 1
+    for (int i = threadIdx.x; i <= tiles_x; i += blockDim.x) edges[i] = (real)(i * tw) / (real)W * 2.0f - 1.0f;
+    for (int i = threadIdx.x; i <= tiles_y; i += blockDim.x) edges[tiles_x + 1 + i] = (real)(i * th) / (real)H * 2.0f - 1.0f;
+    if (threadIdx.x < 2) total_and_status[threadIdx.x] = 0;
+}
+
+__global__ __launch_bounds__(kScanThreads) void bin_setup_kernel(const real4 *__restrict__ vertices, int n_vertices,
+                                                                 const int32_t *__restrict__ indices, int n_triangles, int W, int H,
+                                                                 int tw, int th, int tiles_x, int tiles_y,
+                                                                 uint32_t *__restrict__ tri_offsets, real4 *__restrict__ records,
+                                                                 uint32_t *total, uint32_t *status, uint32_t *ticket, uint64_t *states,
+                                                                 int n_scan_tiles, uint32_t head_capacity, uint32_t *__restrict__ heads) {
+    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_wave_total[kScanThreads / kWave];
+    __shared__ uint32_t s_tile_prefix;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
+    __syncthreads();
+    const int tile = (int)s_tile;
+    const int64_t base = (int64_t)tile * kScanTile + (int64_t)tid * 4;
+
+    uint32_t x[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int64_t t = base + k;
+        if (t >= n_triangles) continue;
+        const TriXYZ p = load_triangle(vertices, n_vertices, indices, (int)t);
+        const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
+        x[k] = rect_count(r);
+        // render.cu:140-152 compute_plane
+        const real det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+        const real id = (real)(1.0 / (double)det);
+        const real A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
+        const real B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
+        const real C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
+        real4 *rec = records + 3 * t;
+        rec[0] = make_real4(A, B, C, int_in_real(r.x0));
+        rec[1] = make_real4(p.ax, p.ay, p.bx, p.by);
+        rec[2] = make_real4(p.cx, p.cy, int_in_real(r.y0), int_in_real(r.y1 - r.y0 + 1));
+    }
+    const uint32_t thread_sum = x[0] + x[1] + x[2] + x[3];
+    const uint32_t incl = wave_inclusive_scan_u32(thread_sum);
+    if (lane == kWave - 1) s_wave_total[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+        uint32_t wt = (lane < kScanThreads / kWave) ? s_wave_total[lane] : 0u;
+        uint32_t wincl = wave_inclusive_scan_u32(wt);
+        uint32_t tile_total = (uint32_t)__builtin_amdgcn_readlane((int)wincl, kScanThreads / kWave - 1);
+        if (lane < kScanThreads / kWave) s_wave_total[lane] = wincl - wt;  // exclusive wave offsets
+        const uint32_t prefix = scan_tile_prefix(states, tile, tile_total, n_scan_tiles, total, status);
+        if (lane == 0) s_tile_prefix = prefix;
+    }
+    __syncthreads();
+    uint32_t run = s_tile_prefix + s_wave_total[wave] + (incl - thread_sum);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int64_t t = base + k;
+        if (t >= n_triangles) break;
+        tri_offsets[t] = run;
+        if (heads && x[k] != 0) {
+            // triangle t owns the key positions [run, run + x): note for every multiple of 256 who owns it
+            const uint32_t first = (run + kBinThreads - 1) / kBinThreads, last = (run + x[k] - 1) / kBinThreads;
+            for (uint32_t h = first; h <= last && h < head_capacity; h++) heads[h] = (uint32_t)t;
+        }
+        run += x[k];
+    }
+}
+
+constexpr int kEdgeWindow = 1024;  // tile edges staged in LDS (more columns + rows than that: read from memory)
+
+// One thread per key, like bin_emit_kernel, from the triangles' records.  A workgroup takes `chunks_per_group`
+// consecutive chunks of 256 keys.  It also counts the digits of the tile passes of the sort that follows (plan,
+// totals: LDS counters, one global atomic per digit and workgroup at the end) and clears zero_words words
+// from `zero` on (the sort's look-back words).
+__global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const real4 *__restrict__ records,
+                                                                       const uint32_t *__restrict__ tri_offsets, int n_triangles,
+                                                                       int64_t n_keys, const uint32_t *__restrict__ owner_heads,
+                                                                       uint32_t owner_capacity, const real *__restrict__ edges,
+                                                                       int tiles_x, int tiles_y, uint64_t *__restrict__ keys,
+                                                                       uint32_t *__restrict__ payload, PassPlan plan,
+                                                                       uint32_t *totals, uint32_t *zero, size_t zero_words,
+                                                                       uint32_t *clear_word, int chunks_per_group) {
+    __shared__ PolyLds lds;
+    __shared__ uint32_t s_offsets[kOwnerWindow];
+    __shared__ real s_edges[kEdgeWindow];
+    __shared__ uint32_t s_hist[kMaxPasses / 2][kRadix];
+    const int tid = threadIdx.x;
+    for (size_t i = (size_t)blockIdx.x * kBinThreads + tid; i < zero_words; i += (size_t)gridDim.x * kBinThreads) zero[i] = 0;
+    if (clear_word && blockIdx.x == 0 && tid == 0) *clear_word = 0;
+    const int n_edges = tiles_x + tiles_y + 2;
+    const bool edges_staged = n_edges <= kEdgeWindow;
+    if (edges_staged)
+        for (int i = tid; i < n_edges; i += kBinThreads) s_edges[i] = edges[i];
+    if (totals)
+        for (int p = 0; p < plan.passes; p++) s_hist[p][tid] = 0;
+    const int64_t n_chunks = (n_keys + kBinThreads - 1) / kBinThreads;
+    const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunks_per_group < n_chunks ? ((int64_t)blockIdx.x + 1) * chunks_per_group : n_chunks;
+    for (int64_t chunk = (int64_t)blockIdx.x * chunks_per_group; chunk < chunk_end; chunk++) {
+        const int64_t k0 = chunk * kBinThreads;
+        const int64_t k = k0 + tid;
+        // The owners of the chunk's 256 keys lie between the owner of its first key and the owner of the next
+        // chunk's first key; the scan noted both (otherwise two uniform binary searches find them).
+        int t_first, t_last;
+        if (owner_heads && chunk < owner_capacity) {
+            t_first = (int)owner_heads[chunk];
+            t_last = (k0 + kBinThreads < n_keys && chunk + 1 < owner_capacity) ? (int)owner_heads[chunk + 1] : n_triangles - 1;
+        } else {
+            const int64_t k_last = (k0 + kBinThreads <= n_keys ? k0 + kBinThreads : n_keys) - 1;
+            t_first = owner_of_key(tri_offsets, n_triangles, (uint32_t)k0);
+            t_last = owner_of_key(tri_offsets, n_triangles, (uint32_t)k_last);
+        }
+        const int span = t_last - t_first + 1;
+        const bool windowed = span <= kOwnerWindow;
+        __syncthreads();  // the previous chunk's searches are done with s_offsets
+        if (windowed)
+            for (int i = tid; i < span; i += kBinThreads) s_offsets[i] = tri_offsets[t_first + i];
+        __syncthreads();
+        if (k >= n_keys) continue;  // the polygon arrays are private per thread; the barriers above are uniform
+
+        int t;
+        uint32_t owner_offset;
+        if (windowed) {
+            int lo = 0, hi = span;  // s_offsets[lo] <= k, answer in [lo, hi)
+            while (hi - lo > 1) {
+                const int mid = lo + ((hi - lo) >> 1);
+                if (s_offsets[mid] <= (uint32_t)k) lo = mid; else hi = mid;
+            }
+            t = t_first + lo;
+            owner_offset = s_offsets[lo];
+        } else {
+            t = owner_of_key(tri_offsets, n_triangles, (uint32_t)k);
+            owner_offset = tri_offsets[t];
+        }
+        const uint32_t local = (uint32_t)k - owner_offset;
+        const real4 r0 = records[3 * (int64_t)t], r1 = records[3 * (int64_t)t + 1], r2 = records[3 * (int64_t)t + 2];
+        const real A = r0.x, B = r0.y, C = r0.z;
+        const uint32_t ny = (uint32_t)int_of_real(r2.w);
+        const int tx = int_of_real(r0.w) + (int)(local / ny);  // tile x outer, tile y inner (render.cu:235-236)
+        const int ty = int_of_real(r2.z) + (int)(local % ny);
+
+        // render.cu:243-246 tile rectangle in NDC
+        real xmin, xmax, ymin, ymax;
+        if (edges_staged) {
+            xmin = s_edges[tx]; xmax = s_edges[tx + 1];
+            ymin = s_edges[tiles_x + 1 + ty]; ymax = s_edges[tiles_x + 2 + ty];
+        } else {
+            xmin = edges[tx]; xmax = edges[tx + 1];
+            ymin = edges[tiles_x + 1 + ty]; ymax = edges[tiles_x + 2 + ty];
+        }
+
+        lds.x[0][0][tid] = r1.x; lds.y[0][0][tid] = r1.y;
+        lds.x[0][1][tid] = r1.z; lds.y[0][1][tid] = r1.w;
+        lds.x[0][2][tid] = r2.x; lds.y[0][2][tid] = r2.y;
+        int n = 3;
+        int cur = 0;  // buffer that holds the current polygon
+        n = clip_pass(lds, cur, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
+        if (n > 0) n = clip_pass(lds, cur, n, -1.0f, 0.0f, -xmax);
+        if (n > 0) n = clip_pass(lds, cur, n, 0.0f, 1.0f, ymin);
+        if (n > 0) n = clip_pass(lds, cur, n, 0.0f, -1.0f, -ymax);
+
+        real key = kFarKey;  // render.cu:259
+        if (n > 0) {
+            real md = std::numeric_limits<real>::max();
+            for (int i = 0; i < n; i++) {
+                const real pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
+                md = (pd < md) ? pd : md;
+            }
+            key = md;
+        }
+        const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
+#ifdef TG_DOUBLE_PRECISION
+        keys[k] = orderable_bits(key);  // all 64 bits are depth; the tile ids follow the depth keys
+        keys[n_keys + k] = tile;
+#else
+        keys[k] = ((uint64_t)tile << 32) | orderable_bits(key);
+#endif
+        payload[k] = (uint32_t)t;
+        if (totals)
+            for (int p = 0; p < plan.passes; p++) atomicAdd(&s_hist[p][(tile >> (plan.shift[p] - 32)) & ((1u << plan.bits[p]) - 1)], 1u);
+    }
+    if (totals) {
+        __syncthreads();
+        for (int p = 0; p < plan.passes; p++) {
+            const uint32_t c = s_hist[p][tid];
+            if (c) atomicAdd(&totals[p * kRadix + tid], c);
+        }
+    }
 }
 
 // Lower bounds of the per-pixel depths (render.cu:404: interpolate3 of the vertex z with the vertex w
@@ -361,16 +584,6 @@ extern "C" int tg_bin_emit(const real *vertices, int32_t n_vertices, const int32
     return check_launch("bin_emit_kernel");
 }
 
-extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int32_t *offsets, void *stream) {
-    if (n_keys < 0 || n_keys > 0x7fffffffll || n_tiles <= 0 || !offsets || (n_keys > 0 && !sorted_keys)) {
-        set_error("tg_tile_ranges: null pointer or size out of range");
-        return TG_E_ARG;
-    }
-    TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n_keys + 1, kBinThreads)), dim3(kBinThreads), 0,
-                       (hipStream_t)stream, sorted_keys, n_keys, n_tiles, offsets);
-    return check_launch("tile_ranges_kernel");
-}
-
 extern "C" int tg_bary(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, real *out,
                        void *stream) {
     if (int e = check_geometry("tg_bary", vertices, n_vertices, indices, n_triangles, 1, 1, 1, 1)) return e;
@@ -403,3 +616,64 @@ extern "C" int tg_list_bounds(const real *vertices, int32_t n_vertices, const in
               sorted_keys, sorted_ids, offsets, bounds, far_start);
     return check_launch("list_bounds_kernel");
 }
+
+extern "C" size_t tg_bin_setup_workspace_bytes(int32_t n_triangles, int width, int height, int tile_w, int tile_h) {
+    if (n_triangles < 0 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0) return 0;
+    return frame_state(nullptr, n_triangles, ceil_div(width, tile_w), ceil_div(height, tile_h)).bytes;
+}
+
+extern "C" int tg_bin_setup(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width,
+                            int height, int tile_w, int tile_h, uint32_t *tri_offsets, real *records, uint32_t *total_and_status,
+                            uint32_t head_capacity, uint32_t *heads, void *frame, size_t frame_bytes, void *stream) {
+    if (int e = check_geometry("tg_bin_setup", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
+    if (!total_and_status || !frame || ((uintptr_t)frame & 255) || (n_triangles > 0 && (!tri_offsets || !records)) ||
+        ((uintptr_t)records & (4 * sizeof(real) - 1))) {
+        set_error("tg_bin_setup: null pointer, frame state not 256-byte aligned or records not aligned to four scalars");
+        return TG_E_ARG;
+    }
+    const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
+    const FrameState f = frame_state(frame, n_triangles, tiles_x, tiles_y);
+    if (frame_bytes < f.bytes) {
+        set_error("tg_bin_setup: frame state of %zu bytes, need %zu", frame_bytes, f.bytes);
+        return TG_E_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int n_scan_tiles = (int)ceil_div64(n_triangles, kScanTile);
+    const size_t zero_words = ((char *)f.edges - (char *)f.tickets) / 4;  // tickets, totals, scan states
+    TG_LAUNCH(bin_init_kernel, dim3(1), dim3(1024), 0, s, f.tickets, zero_words, f.edges, width, height, tile_w, tile_h, tiles_x,
+              tiles_y, total_and_status);
+    if (int e = check_launch("bin_init_kernel")) return e;
+    if (n_triangles == 0) return 0;
+    static int resident_cache[kMaxDevices] = {0};
+    uint32_t *ticket = f.tickets;
+    if (n_scan_tiles <= resident_workgroups((const void *)bin_setup_kernel, kScanThreads, resident_cache)) ticket = nullptr;
+    TG_LAUNCH(bin_setup_kernel, dim3(n_scan_tiles), dim3(kScanThreads), 0, s, (const real4 *)vertices, n_vertices, indices, n_triangles,
+              width, height, tile_w, tile_h, tiles_x, tiles_y, tri_offsets, (real4 *)records, total_and_status, total_and_status + 1,
+              ticket, f.states, n_scan_tiles, head_capacity, heads);
+    return check_launch("bin_setup_kernel");
+}
+
+namespace tg {
+// Launches the emission from records; with `sort_workspace` it also prepares the tile-list sort that follows
+// (digit totals into the frame state, look-back words cleared).
+int launch_emit_records(const char *fn, const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
+                        uint32_t owner_capacity, const uint32_t *owner_heads, void *frame, int width, int height, int tile_w,
+                        int tile_h, uint64_t *keys, uint32_t *payload, uint32_t *zero, size_t zero_words, uint32_t *clear_word,
+                        bool count_digits, hipStream_t s) {
+    const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
+    const FrameState f = frame_state(frame, n_triangles, tiles_x, tiles_y);
+    const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
+    const int64_t n_chunks = ceil_div64(n_keys, kBinThreads);
+    // enough workgroups to fill the device several times over, few enough that the digit totals cost
+    // one atomic per digit and workgroup
+    int chunks_per_group = (int)ceil_div64(n_chunks, 2048);
+    if (chunks_per_group < 1) chunks_per_group = 1;
+    const unsigned grid = (unsigned)ceil_div64(n_chunks, chunks_per_group);
+    TG_LAUNCH(bin_emit_records_kernel, dim3(grid), dim3(kBinThreads), 0, s, (const real4 *)records, tri_offsets, n_triangles, n_keys,
+              owner_heads, owner_capacity, f.edges, tiles_x, tiles_y, keys, payload, plan, count_digits ? f.totals : (uint32_t *)nullptr,
+              zero, zero_words, clear_word, chunks_per_group);
+    return check_launch(fn);
+}
+uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y) { return frame_state(frame, n_triangles, tiles_x, tiles_y).tickets + kStateTicketWords; }
+uint32_t *frame_tickets(void *frame) { return (uint32_t *)frame; }
+}  // namespace tg

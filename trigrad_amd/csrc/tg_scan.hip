@@ -16,21 +16,9 @@
 // wrong result) so that every wave still exits.
 #include <mutex>
 
-#include "tg_common.hpp"
+#include "tg_scan.hpp"
 
 namespace tg {
-
-constexpr int kScanThreads = 512;
-constexpr int kScanTile = kScanThreads * 4;
-constexpr uint32_t kSpinLimit = 1u << 20;
-
-constexpr uint64_t kFlagAggregate = 1ull << 62;
-constexpr uint64_t kFlagInclusive = 2ull << 62;
-
-__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
-    v = wave_inclusive_scan_u32(v);
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
 
 __global__ void scan_init_kernel(uint32_t *ticket, uint64_t *states, int n_tiles, uint32_t *total, uint32_t *status) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -78,38 +66,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_lookback_kernel(const uint3
         uint32_t tile_total = (uint32_t)__builtin_amdgcn_readlane((int)wincl, kScanThreads / kWave - 1);
         if (lane < kScanThreads / kWave) s_wave_total[lane] = wincl - wt;  // exclusive wave offsets
 
-        if (lane == 0) {
-            uint64_t word = (tile == 0 ? kFlagInclusive : kFlagAggregate) | tile_total;
-            __hip_atomic_store(&states[tile], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        uint32_t prefix = 0;
-        bool timed_out = false;
-        for (int look = tile - 1; look >= 0; look -= kWave) {
-            const int idx = look - lane;
-            uint64_t word = kFlagInclusive;  // before the first tile: inclusive prefix 0
-            if (idx >= 0) {
-                uint32_t spins = 0;
-                word = __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                while ((word >> 62) == 0 && spins < kSpinLimit) {
-                    __builtin_amdgcn_s_sleep(1);
-                    word = __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    spins++;
-                }
-                if ((word >> 62) == 0) timed_out = true;
-            }
-            const uint64_t inclusive_lanes = __builtin_amdgcn_ballot_w64((word >> 62) == 2);
-            const int first = inclusive_lanes ? __builtin_ctzll(inclusive_lanes) : kWave;
-            prefix += wave_sum(lane <= first ? (uint32_t)word : 0u);
-            if (inclusive_lanes) break;
-        }
-        if (__builtin_amdgcn_ballot_w64(timed_out) && lane == 0 && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
-        if (lane == 0) {
-            if (tile != 0)
-                __hip_atomic_store(&states[tile], kFlagInclusive | (uint64_t)(prefix + tile_total), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            s_tile_prefix = prefix;
-            if (tile == n_tiles - 1) *total = prefix + tile_total;
-        }
+        const uint32_t prefix = scan_tile_prefix(states, tile, tile_total, n_tiles, total, status);
+        if (lane == 0) s_tile_prefix = prefix;
     }
     __syncthreads();
 

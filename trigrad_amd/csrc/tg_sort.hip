@@ -29,46 +29,9 @@
 // (then no workgroup has to finish for another to start), by the workgroup ids,
 // which saves the serialised same-address atomics.  Waits are bounded
 // (TG_STATUS_LOOKBACK_TIMEOUT).
-#include "tg_common.hpp"
+#include "tg_sort_plan.hpp"
 
 namespace tg {
-
-constexpr int kRadixBits = 8;
-constexpr int kRadix = 1 << kRadixBits;
-constexpr int kMaxPasses = 8;
-constexpr int kSortThreads = 256;
-constexpr int kSortWaves = kSortThreads / kWave;
-constexpr int kSortItems = 16;
-constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
-constexpr int kHistBlocksMax = 256;
-constexpr int kBasesThreads = 1024;
-constexpr int kLookWindow = 4;  // predecessors read per round trip; wider windows only add L2 traffic (measured 1..64)
-constexpr uint32_t kSortSpinLimit = 1u << 20;
-constexpr uint32_t kLbAggregate = 1u << 30;
-constexpr uint32_t kLbInclusive = 2u << 30;
-constexpr uint32_t kLbValueMask = (1u << 30) - 1;
-constexpr int64_t kSortMaxN = (1ll << 30) - 1;
-
-struct SortLayout {
-    int passes;
-    int n_tiles;
-    int hist_blocks;
-    size_t off_tickets, off_partials, off_bases, off_lookback, total;
-};
-
-static SortLayout sort_layout(int64_t n, int end_bit) {
-    SortLayout L;
-    L.passes = end_bit <= 0 ? 0 : (end_bit + kRadixBits - 1) / kRadixBits;
-    L.n_tiles = (int)ceil_div64(n, kSortTile);
-    L.hist_blocks = L.n_tiles < kHistBlocksMax ? (L.n_tiles > 0 ? L.n_tiles : 1) : kHistBlocksMax;
-    size_t o = 0;
-    L.off_bases = o;    o += (size_t)kMaxPasses * kRadix * 4;
-    L.off_partials = o; o += (size_t)kHistBlocksMax * kMaxPasses * kRadix * 4;
-    L.off_tickets = o;  o += 256;  // kMaxPasses tickets, padded; zeroed together with the look-back words
-    L.off_lookback = o; o += (size_t)kMaxPasses * (size_t)(L.n_tiles > 0 ? L.n_tiles : 1) * kRadix * 4;
-    L.total = o;
-    return L;
-}
 
 __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -78,7 +41,7 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
 
 // Also clears `zero_words` words from `zero` on (the tickets and look-back words of the sweeps that
 // follow), a slice per workgroup: a launch of its own for that costs more than the stores.
-__global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, int passes,
+__global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, PassPlan plan,
                                                                       uint32_t *__restrict__ partials, uint32_t *__restrict__ zero,
                                                                       size_t zero_words) {
     for (size_t i = (size_t)blockIdx.x * kSortThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kSortThreads) zero[i] = 0;
@@ -86,6 +49,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint
     // atomics to one address serialise
     __shared__ uint32_t s_hist_wave[kSortWaves][kMaxPasses][kRadix];
     const int tid = threadIdx.x;
+    const int passes = plan.passes;
     uint32_t (*s_hist)[kRadix] = s_hist_wave[tid / kWave];
     for (int w = 0; w < kSortWaves; w++)
         for (int p = 0; p < passes; p++) s_hist_wave[w][p][tid] = 0;
@@ -98,7 +62,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint
 #pragma unroll
         for (int u = 0; u < 4; u++)
             if (i + u * kSortThreads < n)
-                for (int p = 0; p < passes; p++) atomicAdd(&s_hist[p][(k[u] >> (p * kRadixBits)) & (kRadix - 1)], 1u);
+                for (int p = 0; p < passes; p++) atomicAdd(&s_hist[p][(uint32_t)(k[u] >> plan.shift[p]) & ((1u << plan.bits[p]) - 1)], 1u);
     }
     __syncthreads();
     uint32_t *out = partials + (size_t)blockIdx.x * kMaxPasses * kRadix;
@@ -146,14 +110,56 @@ __device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
     return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
+// Stable rank of each of a lane's ITEMS digits among the equal digits of its wave, items in order, lanes in
+// order within an item.  Match: BITS ballots leave in `peers` the lanes that hold the same digit.  The lowest
+// lane of each group adds the group size to the wave's counter row with a returning LDS atomic; LDS serves a
+// wave's instructions in order, so item i sees the counts of items < i, and the atomics are in flight
+// together.  The group reads its leader's result with ds_bpermute.  Afterwards wave_row[d] = the wave's
+// number of digits d.
+template <int BITS, int ITEMS>
+__device__ __forceinline__ void wave_match_rank(const uint32_t (&digit)[ITEMS], uint32_t *wave_row, uint32_t (&rank)[ITEMS]) {
+    constexpr int kGroup = ITEMS < 16 ? ITEMS : 16;  // atomics in flight together
+    static_assert(ITEMS % kGroup == 0, "whole groups");
+#pragma unroll
+    for (int g = 0; g < ITEMS; g += kGroup) {
+        uint32_t below[kGroup];
+        uint32_t leader[kGroup];
+        uint32_t before[kGroup];
+#pragma unroll
+        for (int i = 0; i < kGroup; i++) {
+            const uint32_t d = digit[g + i];
+            uint64_t peers = ~0ull;
+#pragma unroll
+            for (int b = 0; b < BITS; b++) {
+                const bool bit = (d >> b) & 1u;
+                const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
+                peers &= bit ? vote : ~vote;
+            }
+            below[i] = lanes_below(peers);
+            leader[i] = (uint32_t)__builtin_ctzll(peers);
+            before[i] = 0;
+            if (below[i] == 0) before[i] = __hip_atomic_fetch_add(wave_row + d, (uint32_t)__builtin_popcountll(peers), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+#pragma unroll
+        for (int i = 0; i < kGroup; i++)
+            rank[g + i] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader[i] << 2), (int)before[i]) + below[i];
+    }
+}
+
+// One pass over digit (key >> shift) & mask, mask < 2^BITS.  `bases`: the exclusive scan of the digit totals,
+// or, with totals_given, the totals themselves (scanned here).
+template <int BITS>
 __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t *__restrict__ keys_in,
                                                                   const uint32_t *__restrict__ vals_in,
                                                                   uint64_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
-                                                                  int64_t n, int shift, const uint32_t *__restrict__ bases,
+                                                                  int64_t n, int shift, uint32_t mask,
+                                                                  const uint32_t *__restrict__ bases, int totals_given,
                                                                   uint32_t *lookback, uint32_t *ticket, uint32_t *status) {
+    constexpr int kDigits = 1 << BITS;
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_global_delta[kRadix];
     __shared__ uint32_t s_scan_wave[kSortWaves];
+    __shared__ uint32_t s_base_wave[kSortWaves];
     // The ranking counters are dead once every pair knows its place in the tile,
     // so they share LDS with the permutation buffer (51 KB: three workgroups per CU).
     __shared__ __align__(16) unsigned char s_raw[kSortTile * 12];
@@ -165,9 +171,22 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
+    const bool owns_digit = tid < kDigits;
     if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
     for (int w = 0; w < kSortWaves; w++) s_wave_count[w][tid] = 0;
+    // this digit's first output position: given, or the exclusive scan of the totals
+    uint32_t base = owns_digit ? bases[tid] : 0u;
+    uint32_t base_incl = 0;
+    if (totals_given) {
+        base_incl = wave_inclusive_scan_u32(base);
+        if (lane == kWave - 1) s_base_wave[wave] = base_incl;
+    }
     __syncthreads();
+    if (totals_given) {
+        uint32_t wave_prefix = 0;
+        for (int w = 0; w < wave; w++) wave_prefix += s_base_wave[w];
+        base = wave_prefix + base_incl - base;
+    }
     const int tile = (int)s_tile;
     const int64_t tile_base = (int64_t)tile * kSortTile;
     const int n_valid = (int)((n - tile_base) < kSortTile ? (n - tile_base) : kSortTile);
@@ -175,6 +194,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     // Wave-striped loads keep memory order = (wave, item, lane) order.
     uint64_t key[kSortItems];
     uint32_t val[kSortItems];
+    uint32_t digit[kSortItems];
     uint32_t rank[kSortItems];
     const int lane_base = wave * (kWave * kSortItems) + lane;
 #pragma unroll
@@ -187,36 +207,9 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
             key[i] = ~0ull;  // padding ranks after every real pair of the tile
             val[i] = 0;
         }
+        digit[i] = (uint32_t)(key[i] >> shift) & mask;
     }
-
-    // Stable rank of each pair among the pairs of its wave with the same digit.
-    // Match: 8 ballots leave in `peers` the lanes that hold the same digit.  The
-    // lowest lane of each group adds the group size to the wave's counter row
-    // with a returning LDS atomic; LDS serves a wave's instructions in order, so
-    // item i sees the counts of items < i, and the 16 atomics are in flight
-    // together.  The group reads its leader's result with ds_bpermute.
-    uint32_t *wave_row = s_wave_count[wave];
-    uint32_t below[kSortItems];
-    uint32_t leader[kSortItems];
-    uint32_t before[kSortItems];
-#pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
-        const uint32_t d = (uint32_t)(key[i] >> shift) & (kRadix - 1);
-        uint64_t peers = ~0ull;
-#pragma unroll
-        for (int b = 0; b < kRadixBits; b++) {
-            const bool bit = (d >> b) & 1u;
-            const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
-            peers &= bit ? vote : ~vote;
-        }
-        below[i] = lanes_below(peers);
-        leader[i] = (uint32_t)__builtin_ctzll(peers);
-        before[i] = 0;
-        if (below[i] == 0) before[i] = __hip_atomic_fetch_add(wave_row + d, (uint32_t)__builtin_popcountll(peers), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-#pragma unroll
-    for (int i = 0; i < kSortItems; i++)
-        rank[i] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader[i] << 2), (int)before[i]) + below[i];
+    wave_match_rank<BITS, kSortItems>(digit, s_wave_count[wave], rank);
     __syncthreads();
 
     // Thread d owns digit d: per-wave exclusive offsets, tile count, look-back.
@@ -227,20 +220,16 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         s_wave_count[w][tid] = digit_count;
         digit_count += c;
     }
-    // real pairs only: padding always carries digit 255
-    const uint32_t published = (tid == kRadix - 1) ? digit_count - (uint32_t)(kSortTile - n_valid) : digit_count;
+    // real pairs only: padding always carries the largest digit
+    const uint32_t published = ((uint32_t)tid == mask) ? digit_count - (uint32_t)(kSortTile - n_valid) : digit_count;
     uint32_t *my_words = lookback + tid;
-    __hip_atomic_store(my_words + (size_t)tile * kRadix, (tile == 0 ? kLbInclusive : kLbAggregate) | published, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+    if (owns_digit)
+        __hip_atomic_store(my_words + (size_t)tile * kDigits, (tile == 0 ? kLbInclusive : kLbAggregate) | published, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
 
     // exclusive scan of the tile's digit counts (padding included: it sits at the end)
     {
-        uint32_t v = digit_count;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const uint32_t up = __shfl_up(v, off, kWave);
-            if (lane >= off) v += up;
-        }
+        const uint32_t v = wave_inclusive_scan_u32(digit_count);
         if (lane == kWave - 1) s_scan_wave[wave] = v;
         __syncthreads();
         uint32_t wave_prefix = 0;
@@ -253,10 +242,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const uint32_t local_start = s_local_start[tid];
     __syncthreads();  // s_local_start is complete
 #pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
-        const uint32_t d = (uint32_t)(key[i] >> shift) & (kRadix - 1);
-        rank[i] += s_local_start[d] + s_wave_count[wave][d];
-    }
+    for (int i = 0; i < kSortItems; i++) rank[i] += s_local_start[digit[i]] + s_wave_count[wave][digit[i]];
     __syncthreads();  // every pair knows its place: the counters may be overwritten
 #pragma unroll
     for (int i = 0; i < kSortItems; i++) {
@@ -266,12 +252,12 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     // While the pairs settle in LDS the predecessors publish their counts.
     uint32_t prefix = 0;
     bool timed_out = false;
-    for (int look = tile - 1; look >= 0 && !timed_out;) {
+    for (int look = tile - 1; owns_digit && look >= 0 && !timed_out;) {
         uint32_t words[kLookWindow];
 #pragma unroll
         for (int k = 0; k < kLookWindow; k++)
             words[k] = (look - k >= 0)
-                           ? __hip_atomic_load(my_words + (size_t)(look - k) * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                           ? __hip_atomic_load(my_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                            : kLbInclusive;  // before the first tile: inclusive prefix 0
         bool done = false;
 #pragma unroll
@@ -281,7 +267,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
             uint32_t spins = 0;
             while ((word >> 30) == 0 && spins < kSortSpinLimit) {
                 __builtin_amdgcn_s_sleep(1);
-                word = __hip_atomic_load(my_words + (size_t)(look - k) * kRadix, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                word = __hip_atomic_load(my_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 spins++;
             }
             if ((word >> 30) == 0) { timed_out = true; continue; }
@@ -291,11 +277,11 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         if (done) break;
         look -= kLookWindow;
     }
-    if (tile != 0)
-        __hip_atomic_store(my_words + (size_t)tile * kRadix, kLbInclusive | ((prefix + published) & kLbValueMask), __ATOMIC_RELAXED,
+    if (owns_digit && tile != 0)
+        __hip_atomic_store(my_words + (size_t)tile * kDigits, kLbInclusive | ((prefix + published) & kLbValueMask), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     if (timed_out && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
-    s_global_delta[tid] = bases[tid] + prefix - local_start;
+    s_global_delta[tid] = base + prefix - local_start;
 
     __syncthreads();
 #pragma unroll
@@ -303,12 +289,436 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         const int pos = i * kSortThreads + tid;
         if (pos < n_valid) {
             const uint64_t k = s_keys[pos];
-            const uint32_t d = (uint32_t)(k >> shift) & (kRadix - 1);
+            const uint32_t d = (uint32_t)(k >> shift) & mask;
             const uint32_t g = s_global_delta[d] + (uint32_t)pos;
             keys_out[g] = k;
             vals_out[g] = s_vals[pos];
         }
     }
+}
+
+// ---- sorting the segments of a key array that is ordered by its high word ----------------------------
+//
+// After the passes over the tile bits every tile's pairs lie together, in emission order.  One workgroup
+// then sorts a segment by its low key word (the depth bits) without leaving the CU: the pairs sit in
+// registers, four 8-bit passes rank them with the same wave match as the sweeps and exchange them through
+// LDS, and a pass whose digit is the same for the whole segment is left out.  A segment longer than the
+// LDS holds is sorted by its workgroup through memory, pass by pass, between the two buffer pairs.
+
+constexpr int kSegWaveItemsMax = 8;                                // segments up to 512 pairs: one wave each, no barriers
+constexpr int kSegWaveCap = kWave * kSegWaveItemsMax;
+constexpr int kSegLargeItems = 32;                                 // up to 8192 pairs in LDS (64 KB: two workgroups per CU)
+constexpr int kSegLargeCap = kSortThreads * kSegLargeItems;
+constexpr int kSegStreamItems = 8;                                 // chunk of the pass through memory
+constexpr int kSegLargeGrid = 512;
+
+struct SegLds {
+    uint32_t count[kSortWaves][kRadix];
+    uint32_t start[kRadix];
+    uint32_t wave_total[kSortWaves];
+    uint32_t varying;
+};
+
+__device__ __forceinline__ uint32_t wave_or_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v |= (uint32_t)__shfl_xor((int)v, off, kWave);
+    return v;
+}
+
+// Ranks the workgroup's 256 * ITEMS digits (wave-striped order: wave, item, lane) and leaves in place[i]
+// the position of item i in digit order.  Two barriers inside; the caller separates calls by one more.
+template <int ITEMS>
+__device__ __forceinline__ void workgroup_digit_places(const uint32_t (&digit)[ITEMS], SegLds &lds, uint32_t (&place)[ITEMS]) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    for (int w = 0; w < kSortWaves; w++) lds.count[w][tid] = 0;
+    __syncthreads();
+    wave_match_rank<kRadixBits, ITEMS>(digit, lds.count[wave], place);
+    __syncthreads();
+    uint32_t run = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++) {
+        const uint32_t c = lds.count[w][tid];
+        lds.count[w][tid] = run;
+        run += c;
+    }
+    const uint32_t incl = wave_inclusive_scan_u32(run);
+    if (lane == kWave - 1) lds.wave_total[wave] = incl;
+    __syncthreads();
+    uint32_t wave_prefix = 0;
+    for (int w = 0; w < wave; w++) wave_prefix += lds.wave_total[w];
+    lds.start[tid] = wave_prefix + incl - run;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) place[i] += lds.start[digit[i]] + lds.count[wave][digit[i]];
+}
+
+// Sorts keys[start, start + n) / vals by the low key word, in place; n <= 256 * ITEMS.
+template <int ITEMS>
+__device__ __forceinline__ void segment_sort_in_lds(uint64_t *keys, uint32_t *vals, int64_t start, int n, SegLds &lds,
+                                                    uint32_t *ex_keys, uint32_t *ex_vals) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    constexpr int kWaveSpan = kWave * ITEMS;
+    uint32_t key[ITEMS], val[ITEMS];
+    const uint64_t first = keys[start];
+    uint32_t varying = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        const int pos = wave * kWaveSpan + i * kWave + lane;
+        if (pos < n) {
+            key[i] = (uint32_t)keys[start + pos];
+            val[i] = vals[start + pos];
+            varying |= key[i] ^ (uint32_t)first;
+        } else {
+            key[i] = ~0u;  // padding: behind every real pair, and a stable sort keeps it there
+            val[i] = 0;
+        }
+    }
+    if (tid == 0) lds.varying = 0;
+    __syncthreads();
+    varying = wave_or_u32(varying);
+    if (lane == 0 && varying) atomicOr(&lds.varying, varying);
+    __syncthreads();
+    varying = lds.varying;
+    if (varying == 0) return;  // all keys equal: the order stays
+    const int last_pass = (31 - __builtin_clz(varying)) >> 3;
+#pragma unroll 1
+    for (int p = 0; p <= last_pass; p++) {
+        const int shift = p * kRadixBits;
+        if (((varying >> shift) & (kRadix - 1)) == 0) continue;  // the whole segment shares this digit
+        uint32_t digit[ITEMS], place[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) digit[i] = (key[i] >> shift) & (kRadix - 1);
+        workgroup_digit_places<ITEMS>(digit, lds, place);
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            ex_keys[place[i]] = key[i];
+            ex_vals[place[i]] = val[i];
+        }
+        __syncthreads();
+        if (p == last_pass) break;
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            const int pos = wave * kWaveSpan + i * kWave + lane;
+            key[i] = ex_keys[pos];
+            val[i] = ex_vals[pos];
+        }
+        __syncthreads();  // everything is read before the next pass writes the exchange buffer
+    }
+    const uint64_t high = first & 0xffffffff00000000ull;
+    for (int pos = tid; pos < n; pos += kSortThreads) {
+        keys[start + pos] = high | ex_keys[pos];
+        vals[start + pos] = ex_vals[pos];
+    }
+}
+
+// ---- one wave per segment ----
+struct WaveSegLds {
+    uint32_t count[kRadix];
+    uint32_t ex_keys[kSegWaveCap], ex_vals[kSegWaveCap];
+};
+
+// Orders the LDS traffic of one wave: LDS serves a wave's instructions in order, so a lane sees what another
+// lane of its wave wrote by an earlier instruction; this keeps the compiler from moving accesses across.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The calling wave sorts keys[start, start + n) / vals by the low key word, in place; n <= 64 * ITEMS.
+template <int ITEMS>
+__device__ __forceinline__ void segment_sort_in_wave(uint64_t *keys, uint32_t *vals, int64_t start, int n, WaveSegLds &lds) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint32_t key[ITEMS], val[ITEMS];
+    const uint64_t first = keys[start];
+    uint32_t varying = 0;
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        const int pos = i * kWave + lane;
+        if (pos < n) {
+            key[i] = (uint32_t)keys[start + pos];
+            val[i] = vals[start + pos];
+            varying |= key[i] ^ (uint32_t)first;
+        } else {
+            key[i] = ~0u;  // padding: behind every real pair, and a stable sort keeps it there
+            val[i] = 0;
+        }
+    }
+    varying = wave_or_u32(varying);
+    if (varying == 0) return;  // all keys equal: the order stays
+    const int last_pass = (31 - __builtin_clz(varying)) >> 3;
+#pragma unroll 1
+    for (int p = 0; p <= last_pass; p++) {
+        const int shift = p * kRadixBits;
+        if (((varying >> shift) & (kRadix - 1)) == 0) continue;  // the whole segment shares this digit
+        uint32_t digit[ITEMS], place[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) digit[i] = (key[i] >> shift) & (kRadix - 1);
+#pragma unroll
+        for (int j = 0; j < kRadix / kWave; j++) lds.count[j * kWave + lane] = 0;
+        wave_lds_sync();
+        wave_match_rank<kRadixBits, ITEMS>(digit, lds.count, place);
+        wave_lds_sync();
+        // exclusive scan of the 256 digit counts: four neighbouring digits per lane
+        {
+            uint32_t c[kRadix / kWave];
+            uint32_t sum = 0;
+#pragma unroll
+            for (int j = 0; j < kRadix / kWave; j++) { c[j] = lds.count[lane * (kRadix / kWave) + j]; sum += c[j]; }
+            uint32_t run = wave_inclusive_scan_u32(sum) - sum;
+#pragma unroll
+            for (int j = 0; j < kRadix / kWave; j++) { lds.count[lane * (kRadix / kWave) + j] = run; run += c[j]; }
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            place[i] += lds.count[digit[i]];
+            lds.ex_keys[place[i]] = key[i];
+            lds.ex_vals[place[i]] = val[i];
+        }
+        wave_lds_sync();
+        if (p == last_pass) break;
+#pragma unroll
+        for (int i = 0; i < ITEMS; i++) {
+            key[i] = lds.ex_keys[i * kWave + lane];
+            val[i] = lds.ex_vals[i * kWave + lane];
+        }
+        wave_lds_sync();
+    }
+    const uint64_t high = first & 0xffffffff00000000ull;
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+        const int pos = i * kWave + lane;
+        if (pos < n) {
+            keys[start + pos] = high | lds.ex_keys[pos];
+            vals[start + pos] = lds.ex_vals[pos];
+        }
+    }
+}
+
+// One wave per segment; segments longer than kSegWaveCap are queued for segment_sort_large_kernel.
+__global__ __launch_bounds__(kSortThreads) void segment_sort_small_kernel(uint64_t *keys, uint32_t *vals,
+                                                                          const int32_t *__restrict__ offsets, int n_segments,
+                                                                          uint32_t *queue_count, uint32_t *queue) {
+    __shared__ WaveSegLds lds_all[kSortWaves];
+    const int seg = blockIdx.x * kSortWaves + threadIdx.x / kWave;
+    if (seg >= n_segments) return;
+    WaveSegLds &lds = lds_all[threadIdx.x / kWave];
+    const int64_t start = offsets[seg];
+    const int n = offsets[seg + 1] - offsets[seg];
+    if (n <= 1) return;
+    if (n > kSegWaveCap) {
+        if ((threadIdx.x & (kWave - 1)) == 0) queue[atomicAdd(queue_count, 1u)] = (uint32_t)seg;
+        return;
+    }
+    switch ((n + kWave - 1) / kWave) {
+    case 1: segment_sort_in_wave<1>(keys, vals, start, n, lds); break;
+    case 2: segment_sort_in_wave<2>(keys, vals, start, n, lds); break;
+    case 3: segment_sort_in_wave<3>(keys, vals, start, n, lds); break;
+    case 4: segment_sort_in_wave<4>(keys, vals, start, n, lds); break;
+    case 5: segment_sort_in_wave<5>(keys, vals, start, n, lds); break;
+    case 6: segment_sort_in_wave<6>(keys, vals, start, n, lds); break;
+    default: segment_sort_in_wave<8>(keys, vals, start, n, lds); break;
+    }
+}
+
+// The workgroup sorts keys[start, start + n) by the low key word through memory: per 8-bit pass a histogram
+// of the segment, then its chunks in order, every pair written to its final place of the pass in the other
+// buffer pair.  The sorted segment ends in (keys, vals).
+__device__ void segment_sort_through_memory(uint64_t *keys, uint32_t *vals, uint64_t *keys_alt, uint32_t *vals_alt, int64_t start,
+                                            int n, SegLds &lds, uint32_t *hist /* [kRadix] */, uint32_t *next /* [kRadix] */) {
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    constexpr int kChunk = kSortThreads * kSegStreamItems;
+    constexpr int kWaveSpan = kWave * kSegStreamItems;
+    uint64_t *src_k = keys, *dst_k = keys_alt;
+    uint32_t *src_v = vals, *dst_v = vals_alt;
+#pragma unroll 1
+    for (int p = 0; p < 4; p++) {
+        const int shift = p * kRadixBits;
+        hist[tid] = 0;
+        __syncthreads();
+        for (int i = tid; i < n; i += kSortThreads) atomicAdd(&hist[(uint32_t)(src_k[start + i] >> shift) & (kRadix - 1)], 1u);
+        __syncthreads();
+        const uint32_t mine = hist[tid];
+        const bool uniform = __syncthreads_or(mine == (uint32_t)n);
+        if (uniform) continue;  // one digit holds the whole segment: the pass would change nothing
+        {
+            const uint32_t incl = wave_inclusive_scan_u32(mine);
+            if (lane == kWave - 1) lds.wave_total[wave] = incl;
+            __syncthreads();
+            uint32_t wave_prefix = 0;
+            for (int w = 0; w < wave; w++) wave_prefix += lds.wave_total[w];
+            next[tid] = wave_prefix + incl - mine;
+        }
+        __syncthreads();
+        for (int c0 = 0; c0 < n; c0 += kChunk) {
+            uint64_t key[kSegStreamItems];
+            uint32_t val[kSegStreamItems], digit[kSegStreamItems], place[kSegStreamItems];
+            int n_pad = 0;
+#pragma unroll
+            for (int i = 0; i < kSegStreamItems; i++) {
+                const int pos = c0 + wave * kWaveSpan + i * kWave + lane;
+                if (pos < n) {
+                    key[i] = src_k[start + pos];
+                    val[i] = src_v[start + pos];
+                    digit[i] = (uint32_t)(key[i] >> shift) & (kRadix - 1);
+                } else {
+                    key[i] = 0;
+                    val[i] = 0;
+                    digit[i] = kRadix - 1;  // padding: last in the chunk, so behind every real pair of its digit
+                }
+            }
+            n_pad = (c0 + kChunk > n) ? c0 + kChunk - n : 0;
+            workgroup_digit_places<kSegStreamItems>(digit, lds, place);
+            // place = position in the chunk's digit order; the pass position is the digit's running start plus
+            // the rank among the chunk's pairs of that digit
+#pragma unroll
+            for (int i = 0; i < kSegStreamItems; i++) {
+                const int pos = c0 + wave * kWaveSpan + i * kWave + lane;
+                if (pos < n) {
+                    const int64_t to = start + next[digit[i]] + (place[i] - lds.start[digit[i]]);
+                    dst_k[to] = key[i];
+                    dst_v[to] = val[i];
+                }
+            }
+            __syncthreads();
+            // the chunk's count of digit d = start[d + 1] - start[d]
+            const uint32_t end = (tid == kRadix - 1) ? (uint32_t)kChunk - (uint32_t)n_pad : lds.start[tid + 1];
+            const uint32_t begin = lds.start[tid];
+            __syncthreads();
+            next[tid] += (end > begin) ? end - begin : 0u;
+            __syncthreads();
+        }
+        // the next pass reads what this one wrote
+        __threadfence();
+        __syncthreads();
+        __threadfence();
+        uint64_t *tk = src_k; src_k = dst_k; dst_k = tk;
+        uint32_t *tv = src_v; src_v = dst_v; dst_v = tv;
+    }
+    if (src_k != keys) {
+        for (int i = tid; i < n; i += kSortThreads) {
+            keys[start + i] = src_k[start + i];
+            vals[start + i] = src_v[start + i];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kSortThreads, 2) void segment_sort_large_kernel(uint64_t *keys, uint32_t *vals, uint64_t *keys_alt,
+                                                                          uint32_t *vals_alt, const int32_t *__restrict__ offsets,
+                                                                          const uint32_t *queue_count, const uint32_t *queue) {
+    __shared__ SegLds lds;
+    __shared__ uint32_t ex_keys[kSegLargeCap], ex_vals[kSegLargeCap];
+    const uint32_t queued = *queue_count;
+    for (uint32_t q = blockIdx.x; q < queued; q += gridDim.x) {
+        const int seg = (int)queue[q];
+        const int64_t start = offsets[seg];
+        const int n = offsets[seg + 1] - offsets[seg];
+        if (n <= kSortThreads * 4)
+            segment_sort_in_lds<4>(keys, vals, start, n, lds, ex_keys, ex_vals);
+        else if (n <= kSortThreads * 8)
+            segment_sort_in_lds<8>(keys, vals, start, n, lds, ex_keys, ex_vals);
+        else if (n <= kSortThreads * 16)
+            segment_sort_in_lds<16>(keys, vals, start, n, lds, ex_keys, ex_vals);
+        else if (n <= kSegLargeCap)
+            segment_sort_in_lds<kSegLargeItems>(keys, vals, start, n, lds, ex_keys, ex_vals);
+        else
+            segment_sort_through_memory(keys, vals, keys_alt, vals_alt, start, n, lds, ex_keys, ex_keys + kRadix);
+        __syncthreads();  // the next segment reuses the LDS
+    }
+}
+
+__global__ __launch_bounds__(kSortThreads) void tile_ranges_kernel(const uint64_t *__restrict__ sorted_keys, int64_t n_keys,
+                                                                   int n_tiles, int32_t *__restrict__ offsets) {
+    const int64_t i = (int64_t)blockIdx.x * kSortThreads + threadIdx.x;
+    if (i > n_keys) return;
+    const int cur = (i < n_keys) ? (int)(sorted_keys[i] >> 32) : n_tiles;
+    const int prev = (i > 0) ? (int)(sorted_keys[i - 1] >> 32) : -1;
+    for (int t = prev + 1; t <= cur && t <= n_tiles; t++) offsets[t] = (int32_t)i;
+}
+
+template <int BITS>
+static void launch_sweep(dim3 grid, hipStream_t s, const uint64_t *kin, const uint32_t *vin, uint64_t *kout, uint32_t *vout,
+                         int64_t n, int shift, uint32_t mask, const uint32_t *bases, int totals_given, uint32_t *lookback,
+                         uint32_t *ticket, uint32_t *status) {
+    hipLaunchKernelGGL(sort_sweep_kernel<BITS>, grid, dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, shift, mask, bases,
+                       totals_given, lookback, ticket, status);
+}
+
+// The sweeps of `plan` over (keys, values) <-> (keys_alt, values_alt).  bases: per pass kRadix words, the
+// exclusive scan of the digit totals or (totals_given) the totals; lookback: per pass n_sort_tiles * kRadix
+// words, zero; tickets: one word per pass, zero.
+static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, const uint32_t *bases, int totals_given,
+                      uint32_t *lookback, uint32_t *tickets, uint64_t *keys, uint32_t *values, uint64_t *keys_alt,
+                      uint32_t *values_alt, int64_t n, uint32_t *status, hipStream_t s) {
+    uint64_t *kin = keys, *kout = keys_alt;
+    uint32_t *vin = values, *vout = values_alt;
+    // 534 same-address ticket atomics cost 6 us per pass; a grid that fits the device whole takes its
+    // tile numbers from the workgroup ids instead
+    static int resident_cache[kMaxDevices] = {0};
+    const bool whole_grid_resident = n_sort_tiles <= resident_workgroups((const void *)sort_sweep_kernel<kRadixBits>, kSortThreads, resident_cache);
+    // one pair of timing events around all passes: a pair per launch would add its own two
+    // microseconds to every 24 us kernel
+    ProfileScope timed("sort_sweep_kernel", s, plan.passes);
+    for (int p = 0; p < plan.passes; p++) {
+        const dim3 grid(n_sort_tiles);
+        const uint32_t mask = (1u << plan.bits[p]) - 1;
+        uint32_t *lb = lookback + (size_t)p * n_sort_tiles * kRadix;
+        uint32_t *ticket = whole_grid_resident ? (uint32_t *)nullptr : tickets + p;
+        const uint32_t *b = bases + p * kRadix;
+        switch (plan.bits[p]) {
+        case 8: launch_sweep<8>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        case 7: launch_sweep<7>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        case 6: launch_sweep<6>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        case 5: launch_sweep<5>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        default: launch_sweep<4>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        }
+        if (int e = check_launch(fn)) return e;
+        uint64_t *tk = kin; kin = kout; kout = tk;
+        uint32_t *tv = vin; vin = vout; vout = tv;
+    }
+    return 0;
+}
+
+// Histogram, bases and the sweeps of `plan`, everything in the workspace laid out by L.
+static int run_passes(const char *fn, const PassPlan &plan, const SortLayout &L, char *ws, uint64_t *keys, uint32_t *values,
+                      uint64_t *keys_alt, uint32_t *values_alt, int64_t n, uint32_t *status, hipStream_t s) {
+    uint32_t *tickets = (uint32_t *)(ws + L.off_tickets);
+    uint32_t *bases = (uint32_t *)(ws + L.off_bases);
+    uint32_t *partials = (uint32_t *)(ws + L.off_partials);
+    uint32_t *lookback = (uint32_t *)(ws + L.off_lookback);
+    // tickets and look-back words (adjacent) start at zero; bases and partials are fully overwritten
+    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, plan, partials, tickets, L.zero_words);
+    if (int e = check_launch("sort_histogram_kernel")) return e;
+    TG_LAUNCH(sort_bases_kernel, dim3(plan.passes), dim3(kBasesThreads), 0, s, partials, L.hist_blocks, bases, status);
+    if (int e = check_launch("sort_bases_kernel")) return e;
+    return run_sweeps(fn, plan, L.n_tiles, bases, 0, lookback, tickets, keys, values, keys_alt, values_alt, n, status, s);
+}
+
+// Tile ranges of keys that are ordered by tile, then every tile's segment sorted by its depth bits in place.
+static int ranges_and_segments(uint64_t *k, uint32_t *v, uint64_t *k_other, uint32_t *v_other, int64_t n, int n_tiles,
+                               int32_t *offsets, uint32_t *queue_count, uint32_t *queue, hipStream_t s) {
+    TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n + 1, kSortThreads)), dim3(kSortThreads), 0, s, k, n, n_tiles, offsets);
+    if (int e = check_launch("tile_ranges_kernel")) return e;
+    TG_LAUNCH(segment_sort_small_kernel, dim3(ceil_div(n_tiles, kSortWaves)), dim3(kSortThreads), 0, s, k, v, offsets, n_tiles,
+              queue_count, queue);
+    if (int e = check_launch("segment_sort_small_kernel")) return e;
+    TG_LAUNCH(segment_sort_large_kernel, dim3(kSegLargeGrid), dim3(kSortThreads), 0, s, k, v, k_other, v_other, offsets,
+              queue_count, queue);
+    return check_launch("segment_sort_large_kernel");
+}
+
+static int check_sort_buffers(const char *fn, const void *keys, const void *values, const void *keys_alt, const void *values_alt,
+                              const void *workspace) {
+    if (!keys || !values || !keys_alt || !values_alt || !workspace) {
+        set_error("%s: null pointer", fn);
+        return TG_E_ARG;
+    }
+    if (((uintptr_t)keys & 7) || ((uintptr_t)keys_alt & 7) || ((uintptr_t)workspace & 255)) {
+        set_error("%s: keys must be 8-byte aligned, workspace 256-byte aligned", fn);
+        return TG_E_ARG;
+    }
+    return 0;
 }
 
 }  // namespace tg
@@ -317,7 +727,7 @@ using namespace tg;
 
 extern "C" size_t tg_sort_workspace_bytes(int64_t n) {
     if (n < 0 || n > kSortMaxN) return 0;
-    return sort_layout(n, 64).total;
+    return sort_layout(n, kMaxPasses, 0).total;
 }
 
 extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
@@ -336,51 +746,136 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
         }
         return 0;
     }
-    if (!keys || !values || !keys_alt || !values_alt || !workspace) {
-        set_error("tg_sort_pairs_u64_u32: null pointer");
-        return TG_E_ARG;
-    }
-    if (((uintptr_t)keys & 7) || ((uintptr_t)keys_alt & 7) || ((uintptr_t)workspace & 255)) {
-        set_error("tg_sort_pairs_u64_u32: keys must be 8-byte aligned, workspace 256-byte aligned");
-        return TG_E_ARG;
-    }
-    const SortLayout L = sort_layout(n, end_bit);
+    if (int e = check_sort_buffers("tg_sort_pairs_u64_u32", keys, values, keys_alt, values_alt, workspace)) return e;
+    const PassPlan plan = plan_passes(0, end_bit);
+    const SortLayout L = sort_layout(n, plan.passes, 0);
     if (workspace_bytes < L.total) {
         set_error("tg_sort_pairs_u64_u32: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
         return TG_E_WORKSPACE;
     }
-    char *ws = (char *)workspace;
-    uint32_t *tickets = (uint32_t *)(ws + L.off_tickets);
-    uint32_t *bases = (uint32_t *)(ws + L.off_bases);
-    uint32_t *partials = (uint32_t *)(ws + L.off_partials);
-    uint32_t *lookback = (uint32_t *)(ws + L.off_lookback);
-
-    // tickets and look-back words (adjacent) start at zero; bases and partials are fully overwritten
-    const size_t fill_words = 64 + (size_t)L.passes * L.n_tiles * kRadix;
-    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, L.passes, partials, tickets, fill_words);
-    if (int e = check_launch("sort_histogram_kernel")) return e;
-    TG_LAUNCH(sort_bases_kernel, dim3(L.passes), dim3(kBasesThreads), 0, s, partials, L.hist_blocks, bases, status);
-    if (int e = check_launch("sort_bases_kernel")) return e;
-
-    uint64_t *kin = keys, *kout = keys_alt;
-    uint32_t *vin = values, *vout = values_alt;
-    // 534 same-address ticket atomics cost 6 us per pass; a grid that fits the device whole takes its
-    // tile numbers from the workgroup ids instead
-    static int resident_cache[kMaxDevices] = {0};
-    const bool whole_grid_resident = L.n_tiles <= resident_workgroups((const void *)sort_sweep_kernel, kSortThreads, resident_cache);
-    {
-        // one pair of timing events around all passes: a pair per launch would add its own two
-        // microseconds to every 24 us kernel
-        ProfileScope timed("sort_sweep_kernel", s, L.passes);
-        for (int p = 0; p < L.passes; p++) {
-            hipLaunchKernelGGL(sort_sweep_kernel, dim3(L.n_tiles), dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, p * kRadixBits,
-                               bases + p * kRadix, lookback + (size_t)p * L.n_tiles * kRadix,
-                               whole_grid_resident ? (uint32_t *)nullptr : tickets + p, status);
-            if (int e = check_launch("sort_sweep_kernel")) return e;
-            uint64_t *tk = kin; kin = kout; kout = tk;
-            uint32_t *tv = vin; vin = vout; vout = tv;
-        }
-    }
-    *result_in_alt = (L.passes & 1);
+    if (int e = run_passes("tg_sort_pairs_u64_u32", plan, L, (char *)workspace, keys, values, keys_alt, values_alt, n, status, s))
+        return e;
+    *result_in_alt = (plan.passes & 1);
     return 0;
+}
+
+extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n_tiles, int32_t *offsets, void *stream) {
+    if (n_keys < 0 || n_keys > 0x7fffffffll || n_tiles <= 0 || !offsets || (n_keys > 0 && !sorted_keys)) {
+        set_error("tg_tile_ranges: null pointer or size out of range");
+        return TG_E_ARG;
+    }
+    TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n_keys + 1, kSortThreads)), dim3(kSortThreads), 0,
+                       (hipStream_t)stream, sorted_keys, n_keys, n_tiles, offsets);
+    return check_launch("tile_ranges_kernel");
+}
+
+extern "C" size_t tg_tile_list_sort_workspace_bytes(int64_t n, int n_tiles) {
+    if (n < 0 || n > kSortMaxN || n_tiles <= 0) return 0;
+    return sort_layout(n, kMaxPasses / 2, n_tiles).total;
+}
+
+extern "C" int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
+                                  int n_tiles, int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status,
+                                  int *result_in_alt, void *stream) {
+    if (n < 0 || n > kSortMaxN || n_tiles <= 0 || !offsets || !result_in_alt) {
+        set_error("tg_sort_tile_lists: n must be in [0, 2^30), n_tiles positive, offsets and result_in_alt given");
+        return TG_E_ARG;
+    }
+    *result_in_alt = 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (n == 0) {
+        // no keys: the thread of key position 0 writes offsets[t] = 0 for every t
+        TG_LAUNCH(tile_ranges_kernel, dim3(1), dim3(kSortThreads), 0, s, keys, n, n_tiles, offsets);
+        if (int e = check_launch("tile_ranges_kernel")) return e;
+        if (status) {
+            TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
+            if (int e = check_launch("fill_zero_kernel")) return e;
+        }
+        return 0;
+    }
+    if (int e = check_sort_buffers("tg_sort_tile_lists", keys, values, keys_alt, values_alt, workspace)) return e;
+    int tile_bits = 1;
+    while (tile_bits < 32 && (1ll << tile_bits) < (int64_t)n_tiles) tile_bits++;
+    const PassPlan plan = plan_passes(32, 32 + tile_bits);
+    const SortLayout L = sort_layout(n, plan.passes, n_tiles);
+    if (workspace_bytes < L.total) {
+        set_error("tg_sort_tile_lists: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
+        return TG_E_WORKSPACE;
+    }
+    char *ws = (char *)workspace;
+    if (int e = run_passes("tg_sort_tile_lists", plan, L, ws, keys, values, keys_alt, values_alt, n, status, s)) return e;
+    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
+    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
+    *result_in_alt = (plan.passes & 1);
+    return ranges_and_segments(k, v, k_other, v_other, n, n_tiles, offsets, (uint32_t *)(ws + L.off_tickets) + kQueueCountWord,
+                               (uint32_t *)(ws + L.off_queue), s);
+}
+
+// ---- emission + tile lists of a frame -----------------------------------------------------------------
+static size_t build_lookback_bytes(int64_t n_keys, int n_tiles) {
+    const PassPlan plan = tile_pass_plan(n_tiles);
+    const int64_t n_sort_tiles = ceil_div64(n_keys, kSortTile);
+    return (size_t)plan.passes * (size_t)(n_sort_tiles > 0 ? n_sort_tiles : 1) * kRadix * 4;
+}
+
+extern "C" size_t tg_build_tile_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
+    if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0) return 0;
+    return build_lookback_bytes(n_keys, n_tiles) + (size_t)n_tiles * 4;
+}
+
+extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
+                                   uint32_t head_capacity, const uint32_t *heads, void *frame, int width, int height, int tile_w,
+                                   int tile_h, uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt,
+                                   int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status, int emit_only,
+                                   int *result_in_alt, void *stream) {
+    if (n_keys < 0 || n_keys > kSortMaxN || n_triangles < 0 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0 || !frame ||
+        !result_in_alt || (!emit_only && !offsets)) {
+        set_error("tg_build_tile_lists: n_keys must be in [0, 2^30), sizes positive, frame state, offsets and result_in_alt given");
+        return TG_E_ARG;
+    }
+    *result_in_alt = 0;
+    hipStream_t s = (hipStream_t)stream;
+    const int n_tiles = ceil_div(width, tile_w) * ceil_div(height, tile_h);
+    if (n_keys == 0) {
+        if (status) {
+            TG_LAUNCH(fill_zero_kernel, dim3(1), dim3(64), 0, s, status, (size_t)1);
+            if (int e = check_launch("fill_zero_kernel")) return e;
+        }
+        if (emit_only) return 0;
+        TG_LAUNCH(tile_ranges_kernel, dim3(1), dim3(kSortThreads), 0, s, keys, n_keys, n_tiles, offsets);
+        return check_launch("tile_ranges_kernel");
+    }
+    if (!records || !tri_offsets || !keys || !values || ((uintptr_t)keys & 7) || ((uintptr_t)records & (4 * sizeof(real) - 1))) {
+        set_error("tg_build_tile_lists: null or misaligned records, offsets, keys or values");
+        return TG_E_ARG;
+    }
+    if (emit_only)
+        return launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads, frame,
+                                   width, height, tile_w, tile_h, keys, values, nullptr, 0, status, false, s);
+    if (sizeof(real) != 4) {
+        set_error("tg_build_tile_lists: the double build's depth keys take all 64 key bits; emit only, then sort by depth and by tile");
+        return TG_E_ARG;
+    }
+    if (int e = check_sort_buffers("tg_build_tile_lists", keys, values, keys_alt, values_alt, workspace)) return e;
+    const size_t lookback_bytes = build_lookback_bytes(n_keys, n_tiles);
+    if (workspace_bytes < lookback_bytes + (size_t)n_tiles * 4) {
+        set_error("tg_build_tile_lists: workspace of %zu bytes, need %zu", workspace_bytes, lookback_bytes + (size_t)n_tiles * 4);
+        return TG_E_WORKSPACE;
+    }
+    uint32_t *lookback = (uint32_t *)workspace;
+    uint32_t *queue = (uint32_t *)((char *)workspace + lookback_bytes);
+    // the emission clears the look-back words and the status word and adds up the tile digits of its keys
+    if (int e = launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads, frame,
+                                    width, height, tile_w, tile_h, keys, values, lookback, lookback_bytes / 4, status, true, s))
+        return e;
+    const PassPlan plan = tile_pass_plan(n_tiles);
+    const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
+    uint32_t *tickets = frame_tickets(frame);
+    if (int e = run_sweeps("tg_build_tile_lists", plan, (int)ceil_div64(n_keys, kSortTile), frame_totals(frame, n_triangles, tiles_x, tiles_y),
+                           1, lookback, tickets + 8, keys, values, keys_alt, values_alt, n_keys, status, s))
+        return e;
+    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
+    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
+    *result_in_alt = (plan.passes & 1);
+    return ranges_and_segments(k, v, k_other, v_other, n_keys, n_tiles, offsets, tickets + kQueueCountWord, queue, s);
 }

@@ -1,0 +1,89 @@
+// tg_sort_plan.hpp -- digit positions and workspace layout of the radix sort, shared by the sort and by the key
+// emission (which counts the tile digits of the keys it writes and clears the sweeps' look-back words).
+#pragma once
+#include "tg_common.hpp"
+
+namespace tg {
+
+constexpr int kRadixBits = 8;  // widest digit
+constexpr int kRadix = 1 << kRadixBits;
+constexpr int kMaxPasses = 8;
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSortItems = 16;
+constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
+constexpr int kHistBlocksMax = 256;
+constexpr int kBasesThreads = 1024;
+constexpr int kLookWindow = 4;  // predecessors read per round trip; wider windows only add L2 traffic (measured 1..64)
+constexpr uint32_t kSortSpinLimit = 1u << 20;
+constexpr uint32_t kLbAggregate = 1u << 30;
+constexpr uint32_t kLbInclusive = 2u << 30;
+constexpr uint32_t kLbValueMask = (1u << 30) - 1;
+constexpr int64_t kSortMaxN = (1ll << 30) - 1;
+
+// The digit positions of a sort on key bits [begin_bit, end_bit): as few passes of at most 8 bits as
+// cover them, of equal width up to one bit (45 bits: 8 8 8 7 7 7; the 13 tile bits of 1920x1080: 7 6).
+struct PassPlan {
+    int passes;
+    int shift[kMaxPasses];
+    int bits[kMaxPasses];
+};
+
+inline PassPlan plan_passes(int begin_bit, int end_bit) {
+    PassPlan plan;
+    const int n_bits = end_bit - begin_bit;
+    plan.passes = n_bits <= 0 ? 0 : (n_bits + kRadixBits - 1) / kRadixBits;
+    int at = begin_bit;
+    for (int p = 0; p < kMaxPasses; p++) {
+        const int width = p < plan.passes ? n_bits / plan.passes + (p < n_bits % plan.passes ? 1 : 0) : 0;
+        plan.shift[p] = at;
+        plan.bits[p] = width;
+        at += width;
+    }
+    return plan;
+}
+
+struct SortLayout {
+    int n_tiles;
+    int hist_blocks;
+    size_t off_tickets, off_partials, off_bases, off_lookback, off_queue, total;
+    size_t zero_words;  // words from off_tickets on that must be zero before the sweeps start
+};
+
+// queue_entries: room for that many segment numbers behind the look-back words (tile list sort only)
+inline SortLayout sort_layout(int64_t n, int passes, int64_t queue_entries) {
+    SortLayout L;
+    L.n_tiles = (int)ceil_div64(n, kSortTile);
+    L.hist_blocks = L.n_tiles < kHistBlocksMax ? (L.n_tiles > 0 ? L.n_tiles : 1) : kHistBlocksMax;
+    size_t o = 0;
+    L.off_bases = o;    o += (size_t)kMaxPasses * kRadix * 4;
+    L.off_partials = o; o += (size_t)kHistBlocksMax * kMaxPasses * kRadix * 4;
+    L.off_tickets = o;  o += 256;  // kMaxPasses tickets, the status of the segment kernels, the queue length; zeroed with the look-back words
+    L.off_lookback = o; o += (size_t)passes * (size_t)(L.n_tiles > 0 ? L.n_tiles : 1) * kRadix * 4;
+    L.zero_words = (o - L.off_tickets) / 4;
+    L.off_queue = o;    o += (size_t)queue_entries * 4;
+    L.total = o;
+    return L;
+}
+constexpr int kQueueCountWord = 32;  // word of the ticket block that counts the queued segments
+
+
+// Key bits that hold a tile number below n_tiles (at least one).
+inline int tile_bits_of(int n_tiles) {
+    int bits = 1;
+    while (bits < 32 && (1ll << bits) < (int64_t)n_tiles) bits++;
+    return bits;
+}
+inline PassPlan tile_pass_plan(int n_tiles) { return plan_passes(32, 32 + tile_bits_of(n_tiles)); }
+
+
+// Key emission from the triangle records of the frame's binning (tg_binning.hip).  With count_digits the
+// kernel adds the tile digits of its keys to the frame state's totals; it clears zero_words words at `zero`.
+int launch_emit_records(const char *fn, const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
+                        uint32_t owner_capacity, const uint32_t *owner_heads, void *frame, int width, int height, int tile_w,
+                        int tile_h, uint64_t *keys, uint32_t *payload, uint32_t *zero, size_t zero_words, uint32_t *clear_word,
+                        bool count_digits, hipStream_t s);
+uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y);
+uint32_t *frame_tickets(void *frame);
+
+}  // namespace tg

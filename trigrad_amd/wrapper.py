@@ -50,20 +50,20 @@ class Renderer(Function):
             ctx.save_for_backward(vertices, indices, colors, opacities)
         else:
             ctx.skipped = False
-            (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume) = _C.render_forward(
+            (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings, resume) = _C._forward_full(
                 vertices, indices, colors, opacities, width, height, tile_width, tile_height, early_stopping_threshold,
                 not record_timing, per_pixel_sort, max_layers)
-            last, last_depth, sort_status, fragments, hit_masks = resume
-            if record_timing and int(sort_status.item()) != 0:
-                raise RuntimeError("tg_sort_pairs_u64_u32: look-back wait timed out")
+            last, last_depth, status_check, fragments, hit_masks = resume
             # private to this Function: where the reverse traversal starts, and the blend order (per-pixel
-            # order, max_layers <= 32) or the hit masks (tile order)
+            # order, max_layers <= 32) or the hit masks (tile order); the list kernels' status word, which the
+            # backward pass looks at before it trusts the lists
             extras = [t for t in (last_depth, fragments, hit_masks) if t is not None]
             ctx.has_last_depth = last_depth is not None
             ctx.has_fragments = fragments is not None
             ctx.has_hit_masks = hit_masks is not None
+            ctx.status_check = status_check
             saved = [vertices, indices, colors, opacities, sorted_ids, offsets, bary_transforms, image, depthmap, final_weights,
-                     ends, last, sort_status]
+                     ends, last]
             ctx.save_for_backward(*saved, *extras)
         if record_timing:
             return image, depthmap, timings
@@ -77,8 +77,8 @@ class Renderer(Function):
             grad_opacities = torch.zeros_like(ctx.saved_tensors[3])
         else:
             saved = ctx.saved_tensors
-            last, sort_status = saved[11], saved[12]
-            extras = list(saved[13:])
+            last = saved[11]
+            extras = list(saved[12:])
             last_depth = extras.pop(0) if ctx.has_last_depth else None
             fragments = extras.pop(0) if ctx.has_fragments else None
             hit_masks = extras.pop(0) if ctx.has_hit_masks else None
@@ -87,7 +87,7 @@ class Renderer(Function):
                 grad_image = torch.zeros_like(saved[7])
             grad_vertices, grad_colors, grad_opacities = _C.render_backward(
                 grad_image, grad_depthmap, *saved[:11], width, height, tile_width, tile_height, threshold, per_pixel_sort,
-                max_layers, resume=(last, last_depth, sort_status, fragments, hit_masks))
+                max_layers, resume=(last, last_depth, ctx.status_check, fragments, hit_masks))
         # one slot per forward argument (wrapper.py:99-112)
         return (grad_vertices, None, grad_colors, grad_opacities, None, None, None, None, None, None, None, None)
 
