@@ -284,3 +284,23 @@ def test_sort_tile_lists_uniform_digits_and_empty(cuda):
     sk, sv, status, offsets = _C.sort_tile_lists(torch.empty((0,), dtype=torch.int64, device=cuda),
                                                  torch.empty((0,), dtype=torch.int32, device=cuda), 300)
     assert sk.numel() == 0 and int(status.item()) == 0 and offsets.tolist() == [0] * 301
+
+
+def test_frame_route_with_more_than_65536_tiles(cuda, oracle):
+    """Three tile passes (2x2 tiles of a 600x500 image: 75 000 tiles): the emission counts no digits, the sort
+    makes its own histogram; results as the stage-by-stage route gives them."""
+    from trigrad_amd import _C, scenes as S
+    scene = S.random_soup(300, 600, 500, seed=12, sigma_px=14.0, varying_w=True)
+    W, H, tw, th = 600, 500, 2, 2
+    d = to_device(scene, cuda)
+    T = _C.num_tiles(W, H, tw, th)
+    assert T > 65536
+    em = oracle.bin_emit(scene["vertices"], scene["indices"], W, H, tw, th)
+    want_keys, want_vals = oracle.sort_pairs_u64(em["keys64"], em["tri"])
+    setup = _C.bin_setup(d["vertices"], d["indices"], W, H, tw, th)
+    K = int(setup["total_and_status"][0].item())
+    assert K == em["keys64"].shape[0]
+    fkeys, fids, fstatus, foffsets = _C.build_tile_lists(setup, K)
+    np.testing.assert_array_equal(u64(fkeys), want_keys)
+    np.testing.assert_array_equal(fids.cpu().numpy(), want_vals)
+    np.testing.assert_array_equal(foffsets.cpu().numpy(), oracle.tile_ranges(want_keys, T))

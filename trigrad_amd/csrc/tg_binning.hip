@@ -49,45 +49,55 @@ __global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const real4 *__r
 constexpr int kPolyCap = 8;
 constexpr int kOwnerWindow = 1024;  // triangle offsets staged per workgroup for the owner search
 struct PolyLds {
-    real x[2][kPolyCap][kBinThreads];
-    real y[2][kPolyCap][kBinThreads];
+    real x[kPolyCap][kBinThreads];
+    real y[kPolyCap][kBinThreads];
 };
 
-// One Sutherland-Hodgman pass (render.cu:159-189) from buffer `src` to `1-src`
-// against nx*x + ny*y - d >= 0.  Returns the new vertex count.  When every
-// vertex is inside, the pass reproduces its input; `src` then stays current
-// (signalled by leaving it unchanged) and no vertex is copied.
-__device__ __forceinline__ int clip_pass(PolyLds &lds, int &src, int n_in, real nx, real ny, real d) {
+// One Sutherland-Hodgman pass (render.cu:159-189) against nx*x + ny*y - d >= 0, in place.  Returns the new
+// vertex count.  The polygon is read into registers first (the loop over the eight slots is unrolled, so
+// they are plain registers and every distance is computed once); the output goes back to the same LDS slots
+// at its own running index.  When every vertex is inside, the pass reproduces its input and nothing is written.
+__device__ __forceinline__ int clip_pass(PolyLds &lds, int n_in, real nx, real ny, real d) {
     const int tid = threadIdx.x;
+    real px[kPolyCap], py[kPolyCap], dist[kPolyCap];
     bool all_in = true;
-    for (int i = 0; i < n_in; i++) all_in = all_in && (nx * lds.x[src][i][tid] + ny * lds.y[src][i][tid] - d >= 0.0f);
+#pragma unroll
+    for (int i = 0; i < kPolyCap; i++) {
+        if (i < n_in) {
+            px[i] = lds.x[i][tid];
+            py[i] = lds.y[i][tid];
+            dist[i] = nx * px[i] + ny * py[i] - d;
+            all_in = all_in && (dist[i] >= 0.0f);
+        }
+    }
     if (all_in) return n_in;
-    const int dst = 1 - src;
     int n_out = 0;
-    real p0x = lds.x[src][n_in - 1][tid], p0y = lds.y[src][n_in - 1][tid];
+    real p0x = lds.x[n_in - 1][tid], p0y = lds.y[n_in - 1][tid];
     real d0 = nx * p0x + ny * p0y - d;
     bool in0 = d0 >= 0.0f;
-    for (int i = 0; i < n_in; i++) {
-        const real p1x = lds.x[src][i][tid], p1y = lds.y[src][i][tid];
-        const real d1 = nx * p1x + ny * p1y - d;
-        const bool in1 = d1 >= 0.0f;
-        // A convex polygon gains at most one vertex per pass (7 after four); the
-        // capacity test only matters for slivers whose in/out pattern alternates
-        // by rounding, where vertices beyond the eighth are dropped.
-        if (in1 != in0 && n_out < kPolyCap) {
-            const real t = d0 / (d0 - d1);
-            lds.x[dst][n_out][tid] = p0x + t * (p1x - p0x);
-            lds.y[dst][n_out][tid] = p0y + t * (p1y - p0y);
-            n_out++;
+#pragma unroll
+    for (int i = 0; i < kPolyCap; i++) {
+        if (i < n_in) {
+            const real p1x = px[i], p1y = py[i];
+            const real d1 = dist[i];
+            const bool in1 = d1 >= 0.0f;
+            // A convex polygon gains at most one vertex per pass (7 after four); the
+            // capacity test only matters for slivers whose in/out pattern alternates
+            // by rounding, where vertices beyond the eighth are dropped.
+            if (in1 != in0 && n_out < kPolyCap) {
+                const real t = d0 / (d0 - d1);
+                lds.x[n_out][tid] = p0x + t * (p1x - p0x);
+                lds.y[n_out][tid] = p0y + t * (p1y - p0y);
+                n_out++;
+            }
+            if (in1 && n_out < kPolyCap) {
+                lds.x[n_out][tid] = p1x;
+                lds.y[n_out][tid] = p1y;
+                n_out++;
+            }
+            p0x = p1x; p0y = p1y; d0 = d1; in0 = in1;
         }
-        if (in1 && n_out < kPolyCap) {
-            lds.x[dst][n_out][tid] = p1x;
-            lds.y[dst][n_out][tid] = p1y;
-            n_out++;
-        }
-        p0x = p1x; p0y = p1y; d0 = d1; in0 = in1;
     }
-    src = dst;
     return n_out;
 }
 
@@ -166,21 +176,20 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
     const real ymin = (real)(ty * th) / (real)H * 2.0f - 1.0f;
     const real ymax = (real)((ty + 1) * th) / (real)H * 2.0f - 1.0f;
 
-    lds.x[0][0][tid] = p.ax; lds.y[0][0][tid] = p.ay;
-    lds.x[0][1][tid] = p.bx; lds.y[0][1][tid] = p.by;
-    lds.x[0][2][tid] = p.cx; lds.y[0][2][tid] = p.cy;
+    lds.x[0][tid] = p.ax; lds.y[0][tid] = p.ay;
+    lds.x[1][tid] = p.bx; lds.y[1][tid] = p.by;
+    lds.x[2][tid] = p.cx; lds.y[2][tid] = p.cy;
     int n = 3;
-    int cur = 0;  // buffer that holds the current polygon
-    n = clip_pass(lds, cur, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
-    if (n > 0) n = clip_pass(lds, cur, n, -1.0f, 0.0f, -xmax);
-    if (n > 0) n = clip_pass(lds, cur, n, 0.0f, 1.0f, ymin);
-    if (n > 0) n = clip_pass(lds, cur, n, 0.0f, -1.0f, -ymax);
+    n = clip_pass(lds, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
+    if (n > 0) n = clip_pass(lds, n, -1.0f, 0.0f, -xmax);
+    if (n > 0) n = clip_pass(lds, n, 0.0f, 1.0f, ymin);
+    if (n > 0) n = clip_pass(lds, n, 0.0f, -1.0f, -ymax);
 
     real key = kFarKey;  // render.cu:259
     if (n > 0) {
         real md = std::numeric_limits<real>::max();
         for (int i = 0; i < n; i++) {
-            const real pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
+            const real pd = A * lds.x[i][tid] + B * lds.y[i][tid] + C;  // render.cu:154-157
             md = (pd < md) ? pd : md;
         }
         key = md;
@@ -206,10 +215,11 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
 // Frame state (caller's memory, tg_bin_setup_workspace_bytes): scan ticket, the sort's tickets and queue
 // length, the digit totals of the tile passes, the NDC edges of the tile columns and rows, the scan's state
 // words.  bin_init_kernel clears it and fills in the edges.
-constexpr int kRecordReals = TG_RECORD_SCALARS;  // A B C x0 | ax ay bx by | cx cy y0 ny
+constexpr int kRecordReals = TG_RECORD_SCALARS;  // three planes of M x 4: A B C x0 | ax ay bx by | cx cy y0 ny
 static_assert(kRecordReals == 12, "three real4 per triangle");
 constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets; kQueueCountWord: queued segments
-constexpr int kStateTotalsWords = (kMaxPasses / 2) * kRadix;
+constexpr int kEmitDigitPasses = 2;  // tile passes whose digits the emission counts (up to 65536 tiles; the caller sees to that)
+constexpr int kStateTotalsWords = kEmitDigitPasses * kRadix * kTotalsStride;
 static_assert(kQueueCountWord < kStateTicketWords, "the queue length lives in the ticket block");
 
 struct FrameState {
@@ -241,15 +251,59 @@ __global__ __launch_bounds__(1024) void bin_init_kernel(uint32_t *zero, size_t z
     if (threadIdx.x < 2) total_and_status[threadIdx.x] = 0;
 }
 
+// Adds the digits of the tile passes (plan: shifts count from key bit 0, the tile number starts at bit 32) of
+// every tile of the calling lane's rectangle to the workgroup's LDS counters.  A rectangle of up to 64 tiles
+// is walked by its lane; larger ones are taken one after the other by the whole wave, 64 tiles at a time, so
+// that a triangle that covers thousands of tiles does not hold its wave up.  All 64 lanes call this.
+constexpr uint32_t kLaneRectTiles = 64;
+__device__ __forceinline__ void count_tile_digits(const Rect &r, uint32_t count, int tiles_x, const PassPlan &plan,
+                                                  uint32_t (*hist)[kRadix]) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int shift0 = plan.shift[0] - 32, shift1 = plan.shift[1] - 32;
+    const uint32_t mask0 = (1u << plan.bits[0]) - 1, mask1 = (1u << plan.bits[1]) - 1;
+    const bool two = plan.passes > 1;
+    if (count > 0 && count <= kLaneRectTiles) {
+        for (int tx = r.x0; tx <= r.x1; tx++)
+            for (int ty = r.y0; ty <= r.y1; ty++) {
+                const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
+                atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
+                if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
+            }
+    }
+    uint64_t large = __builtin_amdgcn_ballot_w64(count > kLaneRectTiles);
+    while (large) {
+        const int src = __builtin_ctzll(large);
+        large &= large - 1;
+        const int x0 = __shfl(r.x0, src, kWave), y0 = __shfl(r.y0, src, kWave);
+        const int ny = __shfl(r.y1, src, kWave) - y0 + 1, nx = __shfl(r.x1, src, kWave) - x0 + 1;
+        // lane l takes the tiles l, l + 64, ... of the rectangle in column-major order (column = tile x)
+        int col = lane / ny, row = lane % ny;
+        const int col_step = kWave / ny, row_step = kWave % ny;
+        while (col < nx) {
+            const uint32_t tile = (uint32_t)((y0 + row) * tiles_x + x0 + col);
+            atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
+            if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
+            col += col_step;
+            row += row_step;
+            if (row >= ny) { row -= ny; col++; }
+        }
+    }
+}
+
 __global__ __launch_bounds__(kScanThreads) void bin_setup_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                                  const int32_t *__restrict__ indices, int n_triangles, int W, int H,
                                                                  int tw, int th, int tiles_x, int tiles_y,
                                                                  uint32_t *__restrict__ tri_offsets, real4 *__restrict__ records,
                                                                  uint32_t *total, uint32_t *status, uint32_t *ticket, uint64_t *states,
-                                                                 int n_scan_tiles, uint32_t head_capacity, uint32_t *__restrict__ heads) {
+                                                                 int n_scan_tiles, uint32_t head_capacity, uint32_t *__restrict__ heads,
+                                                                 PassPlan plan, uint32_t *totals) {
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_wave_total[kScanThreads / kWave];
     __shared__ uint32_t s_tile_prefix;
+    __shared__ uint32_t s_count[kScanTile];
+    __shared__ uint32_t s_hist[kEmitDigitPasses][kRadix];
+    if (totals && threadIdx.x < kRadix)
+        for (int p = 0; p < kEmitDigitPasses; p++) s_hist[p][threadIdx.x] = 0;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -258,25 +312,41 @@ __global__ __launch_bounds__(kScanThreads) void bin_setup_kernel(const real4 *__
     const int tile = (int)s_tile;
     const int64_t base = (int64_t)tile * kScanTile + (int64_t)tid * 4;
 
-    uint32_t x[4] = {0, 0, 0, 0};
+    // Triangle by triangle across the lanes (neighbouring lanes take neighbouring triangles, so the index
+    // loads and the record stores of a wave are contiguous); the counts then change hands through LDS so that
+    // every thread scans four consecutive ones.
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        const int64_t t = base + k;
-        if (t >= n_triangles) continue;
-        const TriXYZ p = load_triangle(vertices, n_vertices, indices, (int)t);
-        const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
-        x[k] = rect_count(r);
-        // render.cu:140-152 compute_plane
-        const real det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
-        const real id = (real)(1.0 / (double)det);
-        const real A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
-        const real B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
-        const real C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
-        real4 *rec = records + 3 * t;
-        rec[0] = make_real4(A, B, C, int_in_real(r.x0));
-        rec[1] = make_real4(p.ax, p.ay, p.bx, p.by);
-        rec[2] = make_real4(p.cx, p.cy, int_in_real(r.y0), int_in_real(r.y1 - r.y0 + 1));
+        const int64_t t = (int64_t)tile * kScanTile + k * kScanThreads + tid;
+        uint32_t count = 0;
+        Rect rect = {0, -1, 0, -1};
+        if (t < n_triangles) {
+            const TriXYZ p = load_triangle(vertices, n_vertices, indices, (int)t);
+            const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
+            count = rect_count(r);
+            // render.cu:140-152 compute_plane
+            const real det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+            const real id = (real)(1.0 / (double)det);
+            const real A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
+            const real B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
+            const real C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
+            records[t] = make_real4(A, B, C, int_in_real(r.x0));
+            records[(int64_t)n_triangles + t] = make_real4(p.ax, p.ay, p.bx, p.by);
+            records[2 * (int64_t)n_triangles + t] = make_real4(p.cx, p.cy, int_in_real(r.y0), int_in_real(r.y1 - r.y0 + 1));
+            rect = r;
+        }
+        s_count[k * kScanThreads + tid] = count;
+        if (totals) count_tile_digits(rect, count, tiles_x, plan, s_hist);
     }
+    __syncthreads();
+    if (totals && tid < kRadix)
+        for (int p = 0; p < plan.passes; p++) {
+            const uint32_t c = s_hist[p][tid];
+            if (c) atomicAdd(&totals[p * kRadix + tid], c);
+        }
+    uint32_t x[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) x[k] = s_count[tid * 4 + k];
     const uint32_t thread_sum = x[0] + x[1] + x[2] + x[3];
     const uint32_t incl = wave_inclusive_scan_u32(thread_sum);
     if (lane == kWave - 1) s_wave_total[wave] = incl;
@@ -305,7 +375,6 @@ __global__ __launch_bounds__(kScanThreads) void bin_setup_kernel(const real4 *__
     }
 }
 
-constexpr int kEdgeWindow = 1024;  // tile edges staged in LDS (more columns + rows than that: read from memory)
 
 // One thread per key, like bin_emit_kernel, from the triangles' records.  A workgroup takes `chunks_per_group`
 // consecutive chunks of 256 keys.  It also counts the digits of the tile passes of the sort that follows (plan,
@@ -316,22 +385,14 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
                                                                        int64_t n_keys, const uint32_t *__restrict__ owner_heads,
                                                                        uint32_t owner_capacity, const real *__restrict__ edges,
                                                                        int tiles_x, int tiles_y, uint64_t *__restrict__ keys,
-                                                                       uint32_t *__restrict__ payload, PassPlan plan,
-                                                                       uint32_t *totals, uint32_t *zero, size_t zero_words,
-                                                                       uint32_t *clear_word, int chunks_per_group) {
+                                                                       uint32_t *__restrict__ payload, uint32_t *zero,
+                                                                       size_t zero_words, uint32_t *clear_word,
+                                                                       int chunks_per_group) {
     __shared__ PolyLds lds;
     __shared__ uint32_t s_offsets[kOwnerWindow];
-    __shared__ real s_edges[kEdgeWindow];
-    __shared__ uint32_t s_hist[kMaxPasses / 2][kRadix];
     const int tid = threadIdx.x;
     for (size_t i = (size_t)blockIdx.x * kBinThreads + tid; i < zero_words; i += (size_t)gridDim.x * kBinThreads) zero[i] = 0;
     if (clear_word && blockIdx.x == 0 && tid == 0) *clear_word = 0;
-    const int n_edges = tiles_x + tiles_y + 2;
-    const bool edges_staged = n_edges <= kEdgeWindow;
-    if (edges_staged)
-        for (int i = tid; i < n_edges; i += kBinThreads) s_edges[i] = edges[i];
-    if (totals)
-        for (int p = 0; p < plan.passes; p++) s_hist[p][tid] = 0;
     const int64_t n_chunks = (n_keys + kBinThreads - 1) / kBinThreads;
     const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunks_per_group < n_chunks ? ((int64_t)blockIdx.x + 1) * chunks_per_group : n_chunks;
     for (int64_t chunk = (int64_t)blockIdx.x * chunks_per_group; chunk < chunk_end; chunk++) {
@@ -371,37 +432,30 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
             owner_offset = tri_offsets[t];
         }
         const uint32_t local = (uint32_t)k - owner_offset;
-        const real4 r0 = records[3 * (int64_t)t], r1 = records[3 * (int64_t)t + 1], r2 = records[3 * (int64_t)t + 2];
+        const real4 r0 = records[t], r1 = records[(int64_t)n_triangles + t], r2 = records[2 * (int64_t)n_triangles + t];
         const real A = r0.x, B = r0.y, C = r0.z;
         const uint32_t ny = (uint32_t)int_of_real(r2.w);
         const int tx = int_of_real(r0.w) + (int)(local / ny);  // tile x outer, tile y inner (render.cu:235-236)
         const int ty = int_of_real(r2.z) + (int)(local % ny);
 
         // render.cu:243-246 tile rectangle in NDC
-        real xmin, xmax, ymin, ymax;
-        if (edges_staged) {
-            xmin = s_edges[tx]; xmax = s_edges[tx + 1];
-            ymin = s_edges[tiles_x + 1 + ty]; ymax = s_edges[tiles_x + 2 + ty];
-        } else {
-            xmin = edges[tx]; xmax = edges[tx + 1];
-            ymin = edges[tiles_x + 1 + ty]; ymax = edges[tiles_x + 2 + ty];
-        }
+        const real xmin = edges[tx], xmax = edges[tx + 1];  // a few hundred scalars that every key reads: they stay in cache
+        const real ymin = edges[tiles_x + 1 + ty], ymax = edges[tiles_x + 2 + ty];
 
-        lds.x[0][0][tid] = r1.x; lds.y[0][0][tid] = r1.y;
-        lds.x[0][1][tid] = r1.z; lds.y[0][1][tid] = r1.w;
-        lds.x[0][2][tid] = r2.x; lds.y[0][2][tid] = r2.y;
+        lds.x[0][tid] = r1.x; lds.y[0][tid] = r1.y;
+        lds.x[1][tid] = r1.z; lds.y[1][tid] = r1.w;
+        lds.x[2][tid] = r2.x; lds.y[2][tid] = r2.y;
         int n = 3;
-        int cur = 0;  // buffer that holds the current polygon
-        n = clip_pass(lds, cur, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
-        if (n > 0) n = clip_pass(lds, cur, n, -1.0f, 0.0f, -xmax);
-        if (n > 0) n = clip_pass(lds, cur, n, 0.0f, 1.0f, ymin);
-        if (n > 0) n = clip_pass(lds, cur, n, 0.0f, -1.0f, -ymax);
+        n = clip_pass(lds, n, 1.0f, 0.0f, xmin);                 // render.cu:254-257
+        if (n > 0) n = clip_pass(lds, n, -1.0f, 0.0f, -xmax);
+        if (n > 0) n = clip_pass(lds, n, 0.0f, 1.0f, ymin);
+        if (n > 0) n = clip_pass(lds, n, 0.0f, -1.0f, -ymax);
 
         real key = kFarKey;  // render.cu:259
         if (n > 0) {
             real md = std::numeric_limits<real>::max();
             for (int i = 0; i < n; i++) {
-                const real pd = A * lds.x[cur][i][tid] + B * lds.y[cur][i][tid] + C;  // render.cu:154-157
+                const real pd = A * lds.x[i][tid] + B * lds.y[i][tid] + C;  // render.cu:154-157
                 md = (pd < md) ? pd : md;
             }
             key = md;
@@ -414,15 +468,6 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
         keys[k] = ((uint64_t)tile << 32) | orderable_bits(key);
 #endif
         payload[k] = (uint32_t)t;
-        if (totals)
-            for (int p = 0; p < plan.passes; p++) atomicAdd(&s_hist[p][(tile >> (plan.shift[p] - 32)) & ((1u << plan.bits[p]) - 1)], 1u);
-    }
-    if (totals) {
-        __syncthreads();
-        for (int p = 0; p < plan.passes; p++) {
-            const uint32_t c = s_hist[p][tid];
-            if (c) atomicAdd(&totals[p * kRadix + tid], c);
-        }
     }
 }
 
@@ -647,31 +692,30 @@ extern "C" int tg_bin_setup(const real *vertices, int32_t n_vertices, const int3
     static int resident_cache[kMaxDevices] = {0};
     uint32_t *ticket = f.tickets;
     if (n_scan_tiles <= resident_workgroups((const void *)bin_setup_kernel, kScanThreads, resident_cache)) ticket = nullptr;
+    // the digits of the sort's tile passes are counted here, where every triangle's tile rectangle is at hand
+    // (the double build sorts differently, and more than 65536 tiles take a third pass: no counts then)
+    const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
+    const bool count_digits = sizeof(real) == 4 && plan.passes <= kEmitDigitPasses;
     TG_LAUNCH(bin_setup_kernel, dim3(n_scan_tiles), dim3(kScanThreads), 0, s, (const real4 *)vertices, n_vertices, indices, n_triangles,
               width, height, tile_w, tile_h, tiles_x, tiles_y, tri_offsets, (real4 *)records, total_and_status, total_and_status + 1,
-              ticket, f.states, n_scan_tiles, head_capacity, heads);
+              ticket, f.states, n_scan_tiles, head_capacity, heads, plan, count_digits ? f.totals : (uint32_t *)nullptr);
     return check_launch("bin_setup_kernel");
 }
 
 namespace tg {
-// Launches the emission from records; with `sort_workspace` it also prepares the tile-list sort that follows
-// (digit totals into the frame state, look-back words cleared).
+// Launches the emission from records; it also clears zero_words words at `zero` (the look-back words of the
+// sort that follows) and *clear_word.
 int launch_emit_records(const char *fn, const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
                         uint32_t owner_capacity, const uint32_t *owner_heads, void *frame, int width, int height, int tile_w,
                         int tile_h, uint64_t *keys, uint32_t *payload, uint32_t *zero, size_t zero_words, uint32_t *clear_word,
-                        bool count_digits, hipStream_t s) {
+                        hipStream_t s) {
     const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
     const FrameState f = frame_state(frame, n_triangles, tiles_x, tiles_y);
-    const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
     const int64_t n_chunks = ceil_div64(n_keys, kBinThreads);
-    // enough workgroups to fill the device several times over, few enough that the digit totals cost
-    // one atomic per digit and workgroup
-    int chunks_per_group = (int)ceil_div64(n_chunks, 2048);
-    if (chunks_per_group < 1) chunks_per_group = 1;
+    const int chunks_per_group = 1;  // more (fewer, longer-lived workgroups) measured slower: 52 against 47 us on 2.2 M keys
     const unsigned grid = (unsigned)ceil_div64(n_chunks, chunks_per_group);
     TG_LAUNCH(bin_emit_records_kernel, dim3(grid), dim3(kBinThreads), 0, s, (const real4 *)records, tri_offsets, n_triangles, n_keys,
-              owner_heads, owner_capacity, f.edges, tiles_x, tiles_y, keys, payload, plan, count_digits ? f.totals : (uint32_t *)nullptr,
-              zero, zero_words, clear_word, chunks_per_group);
+              owner_heads, owner_capacity, f.edges, tiles_x, tiles_y, keys, payload, zero, zero_words, clear_word, chunks_per_group);
     return check_launch(fn);
 }
 uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y) { return frame_state(frame, n_triangles, tiles_x, tiles_y).tickets + kStateTicketWords; }

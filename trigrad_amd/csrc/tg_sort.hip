@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
     for (int w = 0; w < kSortWaves; w++) s_wave_count[w][tid] = 0;
     // this digit's first output position: given, or the exclusive scan of the totals
-    uint32_t base = owns_digit ? bases[tid] : 0u;
+    uint32_t base = owns_digit ? bases[totals_given ? tid * kTotalsStride : tid] : 0u;
     uint32_t base_incl = 0;
     if (totals_given) {
         base_incl = wave_inclusive_scan_u32(base);
@@ -665,7 +665,7 @@ static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, co
         const uint32_t mask = (1u << plan.bits[p]) - 1;
         uint32_t *lb = lookback + (size_t)p * n_sort_tiles * kRadix;
         uint32_t *ticket = whole_grid_resident ? (uint32_t *)nullptr : tickets + p;
-        const uint32_t *b = bases + p * kRadix;
+        const uint32_t *b = bases + (size_t)p * kRadix * (totals_given ? kTotalsStride : 1);
         switch (plan.bits[p]) {
         case 8: launch_sweep<8>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
         case 7: launch_sweep<7>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
@@ -774,6 +774,26 @@ extern "C" size_t tg_tile_list_sort_workspace_bytes(int64_t n, int n_tiles) {
     return sort_layout(n, kMaxPasses / 2, n_tiles).total;
 }
 
+// (keys, values): n > 0 pairs in any order -> tile passes with a histogram of their own, ranges, segments.
+static int sort_tile_lists_run(const char *fn, uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
+                               int n_tiles, int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status,
+                               int *result_in_alt, hipStream_t s) {
+    if (int e = check_sort_buffers(fn, keys, values, keys_alt, values_alt, workspace)) return e;
+    const PassPlan plan = tile_pass_plan(n_tiles);
+    const SortLayout L = sort_layout(n, plan.passes, n_tiles);
+    if (workspace_bytes < L.total) {
+        set_error("%s: workspace of %zu bytes, need %zu", fn, workspace_bytes, L.total);
+        return TG_E_WORKSPACE;
+    }
+    char *ws = (char *)workspace;
+    if (int e = run_passes(fn, plan, L, ws, keys, values, keys_alt, values_alt, n, status, s)) return e;
+    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
+    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
+    *result_in_alt = (plan.passes & 1);
+    return ranges_and_segments(k, v, k_other, v_other, n, n_tiles, offsets, (uint32_t *)(ws + L.off_tickets) + kQueueCountWord,
+                               (uint32_t *)(ws + L.off_queue), s);
+}
+
 extern "C" int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
                                   int n_tiles, int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status,
                                   int *result_in_alt, void *stream) {
@@ -793,22 +813,8 @@ extern "C" int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *ke
         }
         return 0;
     }
-    if (int e = check_sort_buffers("tg_sort_tile_lists", keys, values, keys_alt, values_alt, workspace)) return e;
-    int tile_bits = 1;
-    while (tile_bits < 32 && (1ll << tile_bits) < (int64_t)n_tiles) tile_bits++;
-    const PassPlan plan = plan_passes(32, 32 + tile_bits);
-    const SortLayout L = sort_layout(n, plan.passes, n_tiles);
-    if (workspace_bytes < L.total) {
-        set_error("tg_sort_tile_lists: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
-        return TG_E_WORKSPACE;
-    }
-    char *ws = (char *)workspace;
-    if (int e = run_passes("tg_sort_tile_lists", plan, L, ws, keys, values, keys_alt, values_alt, n, status, s)) return e;
-    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
-    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
-    *result_in_alt = (plan.passes & 1);
-    return ranges_and_segments(k, v, k_other, v_other, n, n_tiles, offsets, (uint32_t *)(ws + L.off_tickets) + kQueueCountWord,
-                               (uint32_t *)(ws + L.off_queue), s);
+    return sort_tile_lists_run("tg_sort_tile_lists", keys, values, keys_alt, values_alt, n, n_tiles, offsets, workspace,
+                               workspace_bytes, status, result_in_alt, s);
 }
 
 // ---- emission + tile lists of a frame -----------------------------------------------------------------
@@ -818,8 +824,13 @@ static size_t build_lookback_bytes(int64_t n_keys, int n_tiles) {
     return (size_t)plan.passes * (size_t)(n_sort_tiles > 0 ? n_sort_tiles : 1) * kRadix * 4;
 }
 
+// The emission counts the digits of at most this many tile passes (65536 tiles); with more tiles the sort
+// makes its own histogram.
+constexpr int kEmitDigitPasses = 2;
+
 extern "C" size_t tg_build_tile_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
     if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0) return 0;
+    if (tile_pass_plan(n_tiles).passes > kEmitDigitPasses) return tg_tile_list_sort_workspace_bytes(n_keys, n_tiles);
     return build_lookback_bytes(n_keys, n_tiles) + (size_t)n_tiles * 4;
 }
 
@@ -851,10 +862,17 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     }
     if (emit_only)
         return launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads, frame,
-                                   width, height, tile_w, tile_h, keys, values, nullptr, 0, status, false, s);
+                                   width, height, tile_w, tile_h, keys, values, nullptr, 0, status, s);
     if (sizeof(real) != 4) {
         set_error("tg_build_tile_lists: the double build's depth keys take all 64 key bits; emit only, then sort by depth and by tile");
         return TG_E_ARG;
+    }
+    if (tile_pass_plan(n_tiles).passes > kEmitDigitPasses) {
+        if (int e = launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads,
+                                        frame, width, height, tile_w, tile_h, keys, values, nullptr, 0, status, s))
+            return e;
+        return sort_tile_lists_run("tg_build_tile_lists", keys, values, keys_alt, values_alt, n_keys, n_tiles, offsets, workspace,
+                                   workspace_bytes, status, result_in_alt, s);
     }
     if (int e = check_sort_buffers("tg_build_tile_lists", keys, values, keys_alt, values_alt, workspace)) return e;
     const size_t lookback_bytes = build_lookback_bytes(n_keys, n_tiles);
@@ -864,9 +882,9 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     }
     uint32_t *lookback = (uint32_t *)workspace;
     uint32_t *queue = (uint32_t *)((char *)workspace + lookback_bytes);
-    // the emission clears the look-back words and the status word and adds up the tile digits of its keys
+    // the emission clears the look-back words and the status word; the digit totals are the binning kernel's
     if (int e = launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads, frame,
-                                    width, height, tile_w, tile_h, keys, values, lookback, lookback_bytes / 4, status, true, s))
+                                    width, height, tile_w, tile_h, keys, values, lookback, lookback_bytes / 4, status, s))
         return e;
     const PassPlan plan = tile_pass_plan(n_tiles);
     const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);

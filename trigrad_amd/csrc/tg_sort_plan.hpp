@@ -65,6 +65,7 @@ inline SortLayout sort_layout(int64_t n, int passes, int64_t queue_entries) {
     L.total = o;
     return L;
 }
+constexpr int kTotalsStride = 1;  // words between two digit totals (a cache line each was tried: the atomics got no faster)
 constexpr int kQueueCountWord = 32;  // word of the ticket block that counts the queued segments
 
 
@@ -77,12 +78,12 @@ inline int tile_bits_of(int n_tiles) {
 inline PassPlan tile_pass_plan(int n_tiles) { return plan_passes(32, 32 + tile_bits_of(n_tiles)); }
 
 
-// Key emission from the triangle records of the frame's binning (tg_binning.hip).  With count_digits the
-// kernel adds the tile digits of its keys to the frame state's totals; it clears zero_words words at `zero`.
+// Key emission from the triangle records of the frame's binning (tg_binning.hip); it clears zero_words words
+// at `zero` and *clear_word.  The frame state's digit totals come from the binning kernel.
 int launch_emit_records(const char *fn, const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
                         uint32_t owner_capacity, const uint32_t *owner_heads, void *frame, int width, int height, int tile_w,
                         int tile_h, uint64_t *keys, uint32_t *payload, uint32_t *zero, size_t zero_words, uint32_t *clear_word,
-                        bool count_digits, hipStream_t s);
+                        hipStream_t s);
 uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y);
 uint32_t *frame_tickets(void *frame);
 
