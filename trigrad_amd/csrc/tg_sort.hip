@@ -111,13 +111,58 @@ __device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
 }
 
 // Stable rank of each of a lane's ITEMS digits among the equal digits of its wave, items in order, lanes in
-// order within an item.  Match: BITS ballots leave in `peers` the lanes that hold the same digit.  The lowest
-// lane of each group adds the group size to the wave's counter row with a returning LDS atomic; LDS serves a
-// wave's instructions in order, so item i sees the counts of items < i, and the atomics are in flight
-// together.  The group reads its leader's result with ds_bpermute.  Afterwards wave_row[d] = the wave's
+// order within an item.  Match: every lane ORs its lane bit into the 64-bit LDS word of its digit and reads the
+// word back: the lanes that hold the same digit (LDS serves a wave's instructions in order, so the read sees
+// all 64 ORs of the instruction before it).  The lowest lane of each group adds the group size to the wave's
+// counter row with a returning LDS atomic -- item i so sees the counts of items < i -- and clears the mask
+// word; the group reads its leader's result with ds_bpermute.  Two sets of mask words take turns, so that the
+// next item's OR and read are under way while this item's words are still in use.
+// masks: 2 * kRadix words, zero on entry and zero again on return.  Afterwards wave_row[d] = the wave's
 // number of digits d.
+constexpr int kMaskWords = 2 * kRadix;
+template <int ITEMS>
+__device__ __forceinline__ void wave_match_rank(const uint32_t (&digit)[ITEMS], uint32_t *wave_row, unsigned long long *masks,
+                                                uint32_t (&rank)[ITEMS]) {
+    constexpr int kGroup = ITEMS < 16 ? ITEMS : 16;  // returning atomics in flight before their results are used
+    static_assert(ITEMS % kGroup == 0, "whole groups");
+    const unsigned long long me = 1ull << (threadIdx.x & (kWave - 1));
+    (void)__hip_atomic_fetch_or(masks + digit[0], me, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    unsigned long long next = __hip_atomic_load(masks + digit[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#pragma unroll
+    for (int g = 0; g < ITEMS; g += kGroup) {
+        uint32_t below[kGroup];
+        uint32_t leader[kGroup];
+        uint32_t before[kGroup];
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            const int i = g + j;
+            const unsigned long long peers = next;
+            unsigned long long *mine = masks + (i & 1) * kRadix + digit[i];
+            if (i + 1 < ITEMS) {
+                unsigned long long *ahead = masks + ((i + 1) & 1) * kRadix + digit[i + 1];
+                (void)__hip_atomic_fetch_or(ahead, me, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                next = __hip_atomic_load(ahead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            below[j] = lanes_below(peers);
+            leader[j] = (uint32_t)__builtin_ctzll(peers);
+            before[j] = 0;
+            if (below[j] == 0) {
+                before[j] = __hip_atomic_fetch_add(wave_row + digit[i], (uint32_t)__builtin_popcountll(peers), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_store(mine, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kGroup; j++)
+            rank[g + j] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader[j] << 2), (int)before[j]) + below[j];
+    }
+}
+
+// The same ranks with the match done by ballots instead of mask words: BITS ballots leave in `peers` the lanes
+// that hold the same digit (about six vector instructions per bit).  No working memory; the segment sorts use
+// it, whose waves keep the LDS busier than the vector units (measured: mask words 41 against ballots 37 us on
+// the 8160 lists of the headline frame; the sweeps gain from the mask words, 21.6 -> 20 us a pass).
 template <int BITS, int ITEMS>
-__device__ __forceinline__ void wave_match_rank(const uint32_t (&digit)[ITEMS], uint32_t *wave_row, uint32_t (&rank)[ITEMS]) {
+__device__ __forceinline__ void wave_match_rank_ballots(const uint32_t (&digit)[ITEMS], uint32_t *wave_row, uint32_t (&rank)[ITEMS]) {
     constexpr int kGroup = ITEMS < 16 ? ITEMS : 16;  // atomics in flight together
     static_assert(ITEMS % kGroup == 0, "whole groups");
 #pragma unroll
@@ -165,6 +210,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     __shared__ __align__(16) unsigned char s_raw[kSortTile * 12];
     uint32_t (*s_wave_count)[kRadix] = reinterpret_cast<uint32_t (*)[kRadix]>(s_raw);
     uint32_t *s_local_start = reinterpret_cast<uint32_t *>(s_raw) + kSortWaves * kRadix;
+    unsigned long long *s_masks = reinterpret_cast<unsigned long long *>(s_raw + 8192);  // kSortWaves sets of kMaskWords
     uint64_t *s_keys = reinterpret_cast<uint64_t *>(s_raw);
     uint32_t *s_vals = reinterpret_cast<uint32_t *>(s_raw + kSortTile * 8);
 
@@ -174,6 +220,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const bool owns_digit = tid < kDigits;
     if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
     for (int w = 0; w < kSortWaves; w++) s_wave_count[w][tid] = 0;
+    for (int j = tid; j < kSortWaves * kMaskWords; j += kSortThreads) s_masks[j] = 0;
     // this digit's first output position: given, or the exclusive scan of the totals
     uint32_t base = owns_digit ? bases[totals_given ? tid * kTotalsStride : tid] : 0u;
     uint32_t base_incl = 0;
@@ -209,7 +256,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         }
         digit[i] = (uint32_t)(key[i] >> shift) & mask;
     }
-    wave_match_rank<BITS, kSortItems>(digit, s_wave_count[wave], rank);
+    wave_match_rank<kSortItems>(digit, s_wave_count[wave], s_masks + wave * kMaskWords, rank);
     __syncthreads();
 
     // Thread d owns digit d: per-wave exclusive offsets, tile count, look-back.
@@ -224,8 +271,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const uint32_t published = ((uint32_t)tid == mask) ? digit_count - (uint32_t)(kSortTile - n_valid) : digit_count;
     uint32_t *my_words = lookback + tid;
     if (owns_digit)
-        __hip_atomic_store(my_words + (size_t)tile * kDigits, (tile == 0 ? kLbInclusive : kLbAggregate) | published, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(my_words + (size_t)tile * kDigits, kLbAggregate | published, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // exclusive scan of the tile's digit counts (padding included: it sits at the end)
     {
@@ -249,37 +295,69 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         s_keys[rank[i]] = key[i];
         s_vals[rank[i]] = val[i];
     }
-    // While the pairs settle in LDS the predecessors publish their counts.
-    uint32_t prefix = 0;
+    // While the pairs settle in LDS the predecessors publish their counts.  Two levels keep the chain of waits
+    // short: the tiles of a group of kLookGroup read each other's counts directly (all published at about
+    // the same time, so one round of loads), the tile that closes a group publishes the group's total, and
+    // the look-back proper (aggregate / inclusive words, a window of loads per round trip) runs over groups.
+    const int group = tile / kLookGroup, group_first = group * kLookGroup;
+    uint32_t *group_words = lookback + (size_t)gridDim.x * kDigits + tid;
+    uint32_t in_group = 0, group_prefix = 0;
     bool timed_out = false;
-    for (int look = tile - 1; owns_digit && look >= 0 && !timed_out;) {
-        uint32_t words[kLookWindow];
+    if (owns_digit) {
+        for (int j0 = group_first; j0 < tile && !timed_out; j0 += kLookWindow) {
+            uint32_t words[kLookWindow];
 #pragma unroll
-        for (int k = 0; k < kLookWindow; k++)
-            words[k] = (look - k >= 0)
-                           ? __hip_atomic_load(my_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                           : kLbInclusive;  // before the first tile: inclusive prefix 0
-        bool done = false;
+            for (int k = 0; k < kLookWindow; k++)
+                words[k] = (j0 + k < tile) ? __hip_atomic_load(my_words + (size_t)(j0 + k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                           : kLbAggregate;
 #pragma unroll
-        for (int k = 0; k < kLookWindow; k++) {
-            if (done || timed_out) continue;
-            uint32_t word = words[k];
-            uint32_t spins = 0;
-            while ((word >> 30) == 0 && spins < kSortSpinLimit) {
-                __builtin_amdgcn_s_sleep(1);
-                word = __hip_atomic_load(my_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                spins++;
+            for (int k = 0; k < kLookWindow; k++) {
+                if (timed_out) continue;
+                uint32_t word = words[k];
+                uint32_t spins = 0;
+                while ((word >> 30) == 0 && spins < kSortSpinLimit) {
+                    __builtin_amdgcn_s_sleep(1);
+                    word = __hip_atomic_load(my_words + (size_t)(j0 + k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    spins++;
+                }
+                if ((word >> 30) == 0) { timed_out = true; continue; }
+                in_group += word & kLbValueMask;
             }
-            if ((word >> 30) == 0) { timed_out = true; continue; }
-            prefix += word & kLbValueMask;
-            if ((word >> 30) == 2) done = true;
         }
-        if (done) break;
-        look -= kLookWindow;
+        const bool closes_group = tile == group_first + kLookGroup - 1 || tile == (int)gridDim.x - 1;
+        if (closes_group)
+            __hip_atomic_store(group_words + (size_t)group * kDigits, (group == 0 ? kLbInclusive : kLbAggregate) | ((in_group + published) & kLbValueMask),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int look = group - 1; look >= 0 && !timed_out;) {
+            uint32_t words[kLookWindow];
+#pragma unroll
+            for (int k = 0; k < kLookWindow; k++)
+                words[k] = (look - k >= 0)
+                               ? __hip_atomic_load(group_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                               : kLbInclusive;  // before the first group: inclusive prefix 0
+            bool done = false;
+#pragma unroll
+            for (int k = 0; k < kLookWindow; k++) {
+                if (done || timed_out) continue;
+                uint32_t word = words[k];
+                uint32_t spins = 0;
+                while ((word >> 30) == 0 && spins < kSortSpinLimit) {
+                    __builtin_amdgcn_s_sleep(1);
+                    word = __hip_atomic_load(group_words + (size_t)(look - k) * kDigits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    spins++;
+                }
+                if ((word >> 30) == 0) { timed_out = true; continue; }
+                group_prefix += word & kLbValueMask;
+                if ((word >> 30) == 2) done = true;
+            }
+            if (done) break;
+            look -= kLookWindow;
+        }
+        if (closes_group && group != 0)
+            __hip_atomic_store(group_words + (size_t)group * kDigits, kLbInclusive | ((group_prefix + in_group + published) & kLbValueMask),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (owns_digit && tile != 0)
-        __hip_atomic_store(my_words + (size_t)tile * kDigits, kLbInclusive | ((prefix + published) & kLbValueMask), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t prefix = group_prefix + in_group;
     if (timed_out && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
     s_global_delta[tid] = base + prefix - local_start;
 
@@ -326,13 +404,13 @@ __device__ __forceinline__ uint32_t wave_or_u32(uint32_t v) {
 }
 
 // Ranks the workgroup's 256 * ITEMS digits (wave-striped order: wave, item, lane) and leaves in place[i]
-// the position of item i in digit order.  Two barriers inside; the caller separates calls by one more.
+// the position of item i in digit order.  Barriers inside; the caller separates calls by one more.
 template <int ITEMS>
 __device__ __forceinline__ void workgroup_digit_places(const uint32_t (&digit)[ITEMS], SegLds &lds, uint32_t (&place)[ITEMS]) {
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     for (int w = 0; w < kSortWaves; w++) lds.count[w][tid] = 0;
     __syncthreads();
-    wave_match_rank<kRadixBits, ITEMS>(digit, lds.count[wave], place);
+    wave_match_rank_ballots<kRadixBits, ITEMS>(digit, lds.count[wave], place);
     __syncthreads();
     uint32_t run = 0;
 #pragma unroll
@@ -457,7 +535,7 @@ __device__ __forceinline__ void segment_sort_in_wave(uint64_t *keys, uint32_t *v
 #pragma unroll
         for (int j = 0; j < kRadix / kWave; j++) lds.count[j * kWave + lane] = 0;
         wave_lds_sync();
-        wave_match_rank<kRadixBits, ITEMS>(digit, lds.count, place);
+        wave_match_rank_ballots<kRadixBits, ITEMS>(digit, lds.count, place);
         wave_lds_sync();
         // exclusive scan of the 256 digit counts: four neighbouring digits per lane
         {
@@ -663,7 +741,7 @@ static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, co
     for (int p = 0; p < plan.passes; p++) {
         const dim3 grid(n_sort_tiles);
         const uint32_t mask = (1u << plan.bits[p]) - 1;
-        uint32_t *lb = lookback + (size_t)p * n_sort_tiles * kRadix;
+        uint32_t *lb = lookback + (size_t)p * lookback_words_per_pass(n_sort_tiles);
         uint32_t *ticket = whole_grid_resident ? (uint32_t *)nullptr : tickets + p;
         const uint32_t *b = bases + (size_t)p * kRadix * (totals_given ? kTotalsStride : 1);
         switch (plan.bits[p]) {
@@ -821,7 +899,7 @@ extern "C" int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *ke
 static size_t build_lookback_bytes(int64_t n_keys, int n_tiles) {
     const PassPlan plan = tile_pass_plan(n_tiles);
     const int64_t n_sort_tiles = ceil_div64(n_keys, kSortTile);
-    return (size_t)plan.passes * (size_t)(n_sort_tiles > 0 ? n_sort_tiles : 1) * kRadix * 4;
+    return (size_t)plan.passes * lookback_words_per_pass(n_sort_tiles > 0 ? n_sort_tiles : 1) * 4;
 }
 
 // The emission counts the digits of at most this many tile passes (65536 tiles); with more tiles the sort

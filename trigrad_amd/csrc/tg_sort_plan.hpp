@@ -14,7 +14,8 @@ constexpr int kSortItems = 16;
 constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
 constexpr int kHistBlocksMax = 256;
 constexpr int kBasesThreads = 1024;
-constexpr int kLookWindow = 4;  // predecessors read per round trip; wider windows only add L2 traffic (measured 1..64)
+constexpr int kLookWindow = 8;  // look-back words a digit's thread reads per round trip
+constexpr int kLookGroup = 32;  // sort tiles whose counts are read directly; the look-back proper runs over groups of them
 constexpr uint32_t kSortSpinLimit = 1u << 20;
 constexpr uint32_t kLbAggregate = 1u << 30;
 constexpr uint32_t kLbInclusive = 2u << 30;
@@ -43,6 +44,11 @@ inline PassPlan plan_passes(int begin_bit, int end_bit) {
     return plan;
 }
 
+// Look-back words of one pass: a row of kRadix per sort tile, then a row per group of tiles.
+inline size_t lookback_words_per_pass(int64_t n_sort_tiles) {
+    return (size_t)(n_sort_tiles + ceil_div64(n_sort_tiles, kLookGroup)) * kRadix;
+}
+
 struct SortLayout {
     int n_tiles;
     int hist_blocks;
@@ -59,7 +65,7 @@ inline SortLayout sort_layout(int64_t n, int passes, int64_t queue_entries) {
     L.off_bases = o;    o += (size_t)kMaxPasses * kRadix * 4;
     L.off_partials = o; o += (size_t)kHistBlocksMax * kMaxPasses * kRadix * 4;
     L.off_tickets = o;  o += 256;  // kMaxPasses tickets, the status of the segment kernels, the queue length; zeroed with the look-back words
-    L.off_lookback = o; o += (size_t)passes * (size_t)(L.n_tiles > 0 ? L.n_tiles : 1) * kRadix * 4;
+    L.off_lookback = o; o += (size_t)passes * lookback_words_per_pass(L.n_tiles > 0 ? L.n_tiles : 1) * 4;
     L.zero_words = (o - L.off_tickets) / 4;
     L.off_queue = o;    o += (size_t)queue_entries * 4;
     L.total = o;
