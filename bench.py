@@ -27,6 +27,7 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+sys.path.insert(1, os.path.join(ROOT, "tests"))  # the seeded scene generators live with the tests
 
 HBM_PEAK_GBS = 8000.0
 
@@ -60,7 +61,8 @@ def main():
     import numpy as np
     import torch
     import trigrad_amd
-    from trigrad_amd import _C, scenes
+    from trigrad_amd import _C
+    import scenes
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -208,6 +210,17 @@ def main():
         sweep_us = total_ms / launches * 1000.0
         extra["sort_standalone"]["sweep_kernel"] = {"avg_launch_us": sweep_us, "GBps": 24.0 * n / (sweep_us * 1e-6) / 1e9,
                                                     "frac_of_hbm_peak": 24.0 * n / (sweep_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        # the one scene the reference publishes a time for (notebooks/renderer.ipynb:79, 93-95: 10.9 ms without and
+        # 11.5 ms with per-pixel sort, forward only, GPU not stated): 500 x 500 staggered grid, opacity 1, 500 x 500 px
+        del kbuf, vbuf, keys0, vals0
+        grid = scenes.grid_mesh(500, 500, -0.9, 0.9, -0.9, 0.9)
+        g = {k: torch.from_numpy(v).to(dev) for k, v in grid.items() if isinstance(v, np.ndarray)}
+        ref_scene = {"triangles": int(grid["indices"].shape[0]), "vertices": int(grid["vertices"].shape[0]),
+                     "reference_notebook_ms": {"per_pixel_sort_false": 10.9, "per_pixel_sort_true": 11.5}}
+        for pps in (False, True):
+            t = timed(lambda: trigrad_amd.render(g["vertices"], g["indices"], g["colors"], g["opacities"], per_pixel_sort=pps), 20, 3)
+            ref_scene[f"forward_ms_per_pixel_sort_{str(pps).lower()}"] = t
+        extra["reference_timing_scene"] = ref_scene
     out["extra"] = extra
 
     if not args.no_cpu_baseline:

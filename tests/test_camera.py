@@ -159,7 +159,7 @@ def test_projected_split_mesh_renders(cuda):
     """A mesh reaching behind the camera renders to finite values after splitting, and
     splitting a mesh that lies wholly in front changes nothing in the image."""
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     W, H = 96, 64
     g = torch.Generator().manual_seed(3)
     pos = torch.randn((90, 3), generator=g) * torch.tensor([1.5, 1.0, 2.5])

@@ -79,7 +79,8 @@ DOUBLE_MODES = {"A": dict(per_pixel_sort=True, max_layers=32), "A_3": dict(per_p
 @pytest.mark.parametrize("name", sorted(DOUBLE_SCENES))
 def test_double_build_matches_oracle(name, mode, cuda, oracle):
     """Lists and bary matrices bit-exact, image bit-identical, gradients to 1e-9 against the oracle's float64 instantiation."""
-    from trigrad_amd import _C, scenes as S
+    from trigrad_amd import _C
+    import scenes as S
     scene, tw, th = DOUBLE_SCENES[name](S)
     scene = _as_double(scene)
     m = DOUBLE_MODES[mode]
@@ -141,7 +142,7 @@ def test_reference_gradcheck_suite(scene, output, wrt, per_pixel_sort, cuda, dou
     """gradcheck(render) with the reference's scenes, sizes (50x50, 4x4 tiles) and threshold; the reference runs
     the default mode only, the tile-order mode is added."""
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     v, i, c, o = _reference_case(S, scene, cuda)
     if "v" in wrt:
         v.requires_grad_()

@@ -25,7 +25,7 @@ _cache = {}
 
 
 def _scene(cfg):
-    from trigrad_amd import scenes as S
+    import scenes as S
     if cfg not in _cache:
         _cache.clear()
         _cache[cfg] = S.config(cfg)

@@ -15,7 +15,8 @@ TILES = [(16, 16), (8, 8), (4, 4), (32, 32), (8, 4), (12, 20), (24, 16), (16, 8)
 @pytest.mark.parametrize("block", range(8))
 def test_random_scenes_match_oracle(block, cuda, oracle):
     import torch
-    from trigrad_amd import _C, scenes as S
+    from trigrad_amd import _C
+    import scenes as S
     for case in range(block * 40, block * 40 + 40):
         rng = np.random.default_rng(1000 + case)
         W, H = int(rng.integers(8, 260)), int(rng.integers(8, 200))

@@ -108,8 +108,6 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
     from trigrad_amd import _C
     scene, tw, th = SCENES[name]()
     m = MODES[mode]
-    if name == "degenerate" and m["per_pixel_sort"]:
-        pytest.skip("scene holds NaN pixel depths; their place in the per-pixel order is parity-unpinned")
     d, want, got, ml = _forward_both(scene, tw, th, m, cuda, oracle)
     W, H = scene["width"], scene["height"]
     gi, gd = _grad_inputs(scene, 5, with_depth)
@@ -153,7 +151,7 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
 def test_default_mode_literal_and_policy_agree(oracle):
     """With per_pixel_sort on and at most 32 blended fragments the literal
     reference traversal and the reverse-order policy are the same computation."""
-    from trigrad_amd import scenes as S
+    import scenes as S
     scene = S.random_soup(300, 64, 64, seed=9, sigma_px=14.0, varying_w=True)
     W = H = 64
     fwd = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H)
@@ -168,7 +166,7 @@ def test_render_autograd_end_to_end(cuda, oracle):
     """trigrad_amd.render + loss.backward() on configuration 0 (both modes)."""
     import torch
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     scene = S.config(0)
     W, H = scene["width"], scene["height"]
     d = to_device(scene, cuda)
@@ -195,7 +193,7 @@ def test_loss_on_depth_only(cuda, oracle):
     """Only the depth map takes part in the loss: the image's gradient arrives as None."""
     import torch
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     scene = S.random_soup(400, 96, 80, seed=21, sigma_px=9.0, varying_w=True)
     W, H = scene["width"], scene["height"]
     d = to_device(scene, cuda)
@@ -221,7 +219,7 @@ def test_repeatable_and_stream_ordered(mode, cuda):
     call on a side stream, ordered after the inputs' producer, gives the same result as on the default stream."""
     import torch
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     if mode not in MODES:
         pytest.skip("mode table changed")
     kw = dict(per_pixel_sort=MODES[mode]["per_pixel_sort"], max_layers=MODES[mode]["max_layers"])
@@ -280,7 +278,8 @@ def test_list_bounds_values(cuda):
     """tg_list_bounds: per tile and 256 entries, min over the rest of the list of (min z - 32 ulp max|z|); -inf where a
     weight is not positive and finite."""
     import torch
-    from trigrad_amd import _C, _lib, scenes as S
+    from trigrad_amd import _C, _lib
+    import scenes as S
     scene = S.random_soup(3000, 64, 48, seed=13, sigma_px=30.0, varying_w=True)
     v = scene["vertices"].copy()
     v[5, 3] = -1.0          # a negative weight
@@ -321,7 +320,7 @@ def test_list_bounds_values(cuda):
 def test_record_timing_and_empty_scene(cuda):
     import torch
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     d = to_device(S.config(0), cuda)
     image, depthmap, timings = trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], 256, 256, record_timing=True)
     assert set(timings) == {"init", "per_tile_lists", "sorting", "bary_transforms", "rasterization"}
@@ -340,7 +339,7 @@ def test_record_timing_and_empty_scene(cuda):
 def test_argument_errors(cuda):
     import torch
     import trigrad_amd
-    from trigrad_amd import scenes as S
+    import scenes as S
     d = to_device(S.config(0), cuda)
     v, i, c, o = d["vertices"], d["indices"], d["colors"], d["opacities"]
     with pytest.raises(ValueError, match="tile_width \\* tile_height must be <= 1024"):
@@ -390,7 +389,7 @@ def test_native_surface_as_the_reference_wrapper_calls_it(mode, drop_private_sta
     """_C.render_forward / _C.render_backward with the reference's argument lists and nothing else carried over:
     with the private state that travels on `ends`, and after a caller lost it (it is then computed again)."""
     import torch
-    from trigrad_amd import scenes as S
+    import scenes as S
     scene = S.random_soup(700, 150, 110, seed=21, sigma_px=11.0, varying_w=True)
     m = MODES[mode]
     W, H = scene["width"], scene["height"]
@@ -422,7 +421,8 @@ def test_expired_wait_is_reported_on_every_path(cuda):
     the status word is forged."""
     import torch
     import trigrad_amd
-    from trigrad_amd import _C, scenes as S
+    from trigrad_amd import _C
+    import scenes as S
     d = to_device(S.config(0), cuda)
     args = (d["vertices"], d["indices"], d["colors"], d["opacities"], 256, 256, 16, 16, 1 / 256)
     *results, resume = _C._forward_full(*args, True, False, 2000)

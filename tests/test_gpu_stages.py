@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _scenes():
-    from trigrad_amd import scenes as S
+    import scenes as S
     out = {
         "config0": lambda: (S.config(0, with_target=False), 16, 16),
         "soup_varying_w": lambda: (S.random_soup(3000, 300, 200, seed=1, sigma_px=9.0, varying_w=True), 16, 16),
@@ -38,7 +38,7 @@ def _scenes():
 
 def _degenerate_scene():
     """Zero-area, NaN, infinite, huge and far off-screen triangles mixed with ordinary ones."""
-    from trigrad_amd import scenes as S
+    import scenes as S
     s = S.random_soup(64, 96, 80, seed=11, sigma_px=10.0, varying_w=True)
     v = s["vertices"].copy()
     v[0:3, :2] = v[0, :2]                       # zero area
@@ -214,7 +214,8 @@ def test_tile_ranges_with_empty_tiles(cuda, oracle):
 def test_out_of_range_indices_are_skipped(cuda):
     """A triangle naming a vertex outside [0, V) counts no tiles instead of being read."""
     import torch
-    from trigrad_amd import _C, scenes as S
+    from trigrad_amd import _C
+    import scenes as S
     s = S.random_soup(10, 64, 64, seed=3)
     idx = s["indices"].copy()
     idx[4, 1] = 10_000
@@ -289,7 +290,8 @@ def test_sort_tile_lists_uniform_digits_and_empty(cuda):
 def test_frame_route_with_more_than_65536_tiles(cuda, oracle):
     """Three tile passes (2x2 tiles of a 600x500 image: 75 000 tiles): the emission counts no digits, the sort
     makes its own histogram; results as the stage-by-stage route gives them."""
-    from trigrad_amd import _C, scenes as S
+    from trigrad_amd import _C
+    import scenes as S
     scene = S.random_soup(300, 600, 500, seed=12, sigma_px=14.0, varying_w=True)
     W, H, tw, th = 600, 500, 2, 2
     d = to_device(scene, cuda)

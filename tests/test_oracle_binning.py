@@ -6,7 +6,7 @@ matrix, sign of a clip plane) fails it."""
 import numpy as np
 import pytest
 
-from trigrad_amd import scenes as S
+import scenes as S
 
 F = np.float32
 

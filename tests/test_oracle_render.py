@@ -19,7 +19,7 @@ import pytest
 import torch
 
 import independent_renderer as IR
-from trigrad_amd import scenes as S
+import scenes as S
 
 D = np.float64
 

@@ -652,14 +652,20 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
 // half the room per scalar and twice the candidate lists)
 constexpr int kAccWindow = sizeof(real) == 4 ? 512 : 128;
 
+// The order the reverse selection walks: by pixel depth, a NaN depth behind every number (that is where the
+// forward selection leaves such a fragment, render.cu:338-373: every comparison with it is false), equal
+// depths (two NaNs count as equal) by list position.
+__device__ __forceinline__ bool depth_before(real a, real b) { return a < b || (b != b && a == a); }
+__device__ __forceinline__ bool depth_same(real a, real b) { return a == b || (a != a && b != b); }
+
 // Candidate insertion for the reverse selection: keeps the `cap` LARGEST
 // (depth, position) pairs in descending order.  Positions arrive in ascending
 // order, so a candidate whose depth equals a stored one has the larger position
 // and goes in front of it.
 __device__ __forceinline__ void topk_insert_desc(const TopK &tk, int cap, int &n, real d, int j) {
-    if (n == cap && d < tk.d(cap - 1)) return;
+    if (n == cap && depth_before(d, tk.d(cap - 1))) return;
     int i = (n < cap) ? n : cap - 1;
-    while (i > 0 && d >= tk.d(i - 1)) {
+    while (i > 0 && !depth_before(d, tk.d(i - 1))) {
         tk.d(i) = tk.d(i - 1);
         tk.j(i) = tk.j(i - 1);
         i--;
@@ -733,7 +739,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 const real pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);
                 const int j = batch + e;
-                if (pd < bound_depth || (pd == bound_depth && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
+                if (depth_before(pd, bound_depth) || (depth_same(pd, bound_depth) && j < bound_j)) topk_insert_desc(tk, cap, found, pd, j);
             }
         }
         if (want) {
