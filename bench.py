@@ -198,6 +198,14 @@ def main():
         t_sort = timed(sort_once, 10, 2) - timed(copy_only, 10, 2)
         extra["sort_standalone"] = {"keys": n, "ms": t_sort, "Gkeys_per_s": n / (t_sort / 1000.0) / 1e9,
                                     "GBps": (8.0 + 24.0 * passes) * n / (t_sort / 1000.0) / 1e9}
+        # the same pairs through the sort the frame uses (tile bits through memory, depth bits per tile in LDS)
+        def tile_sort_once():
+            kbuf.copy_(keys0)
+            vbuf.copy_(vals0)
+            _C.sort_tile_lists(kbuf, vbuf, T)
+        t_tile = timed(tile_sort_once, 10, 2) - timed(copy_only, 10, 2)
+        extra["tile_list_sort_standalone"] = {"keys": n, "tiles": T, "ms": t_tile, "Gkeys_per_s": n / (t_tile / 1000.0) / 1e9,
+                                              "note": "same sorted keys, values and tile ranges as the 45-bit sort + tg_tile_ranges"}
         # the sweep kernel alone at this size, from the library's events: 24 bytes per pair and launch
         _C.profile_enable(True)
         _C.profile_report()

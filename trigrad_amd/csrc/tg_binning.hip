@@ -212,15 +212,13 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
 // corners.  bin_emit_records_kernel then reads one record per key instead of the triangle's indices and
 // vertices, and does per key only what depends on the tile: the clip and the minimum.
 //
-// Frame state (caller's memory, tg_bin_setup_workspace_bytes): scan ticket, the sort's tickets and queue
-// length, the digit totals of the tile passes, the NDC edges of the tile columns and rows, the scan's state
-// words.  bin_init_kernel clears it and fills in the edges.
+// Frame state (caller's memory, tg_bin_setup_workspace_bytes): scan ticket, the sort's tickets, the digit
+// totals of the tile passes, the NDC edges of the tile columns and rows, the scan's state words.  bin_init_kernel clears it and fills in the edges.
 constexpr int kRecordReals = TG_RECORD_SCALARS;  // three planes of M x 4: A B C x0 | ax ay bx by | cx cy y0 ny
 static_assert(kRecordReals == 12, "three real4 per triangle");
-constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets; kQueueCountWord: queued segments
+constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets
 constexpr int kEmitDigitPasses = 2;  // tile passes whose digits the emission counts (up to 65536 tiles; the caller sees to that)
 constexpr int kStateTotalsWords = kEmitDigitPasses * kRadix * kTotalsStride;
-static_assert(kQueueCountWord < kStateTicketWords, "the queue length lives in the ticket block");
 
 struct FrameState {
     uint32_t *tickets;

@@ -41,36 +41,38 @@ __global__ void fill_zero_kernel(uint32_t *p, size_t n_words) {
 
 // Also clears `zero_words` words from `zero` on (the tickets and look-back words of the sweeps that
 // follow), a slice per workgroup: a launch of its own for that costs more than the stores.
-__global__ __launch_bounds__(kSortThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, PassPlan plan,
+// 1024 threads a workgroup (one per CU at most 256 workgroups: the partials stay few) keep the LDS atomics of
+// sixteen waves in flight; the counters exist once per pair of waves, because the upper passes see few
+// distinct digits (the tile bits) and LDS atomics to one address serialise.
+constexpr int kHistThreads = 1024;
+constexpr int kHistSets = kHistThreads / kWave / 2;
+__global__ __launch_bounds__(kHistThreads) void sort_histogram_kernel(const uint64_t *__restrict__ keys, int64_t n, PassPlan plan,
                                                                       uint32_t *__restrict__ partials, uint32_t *__restrict__ zero,
                                                                       size_t zero_words) {
-    for (size_t i = (size_t)blockIdx.x * kSortThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kSortThreads) zero[i] = 0;
-    // one set of counters per wave: the upper passes see few distinct digits (the tile bits), and LDS
-    // atomics to one address serialise
-    __shared__ uint32_t s_hist_wave[kSortWaves][kMaxPasses][kRadix];
+    for (size_t i = (size_t)blockIdx.x * kHistThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kHistThreads) zero[i] = 0;
+    __shared__ uint32_t s_hist_set[kHistSets][kMaxPasses][kRadix];
     const int tid = threadIdx.x;
     const int passes = plan.passes;
-    uint32_t (*s_hist)[kRadix] = s_hist_wave[tid / kWave];
-    for (int w = 0; w < kSortWaves; w++)
-        for (int p = 0; p < passes; p++) s_hist_wave[w][p][tid] = 0;
+    uint32_t (*s_hist)[kRadix] = s_hist_set[tid / (2 * kWave)];
+    for (int j = tid; j < kHistSets * kMaxPasses * kRadix; j += kHistThreads) s_hist_set[0][0][j] = 0;
     __syncthreads();
-    const int64_t stride = (int64_t)gridDim.x * kSortThreads * 4;
-    for (int64_t i = (int64_t)blockIdx.x * kSortThreads * 4 + tid; i < n; i += stride) {
+    const int64_t stride = (int64_t)gridDim.x * kHistThreads * 4;
+    for (int64_t i = (int64_t)blockIdx.x * kHistThreads * 4 + tid; i < n; i += stride) {
         uint64_t k[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) k[u] = (i + u * kSortThreads < n) ? keys[i + u * kSortThreads] : 0;
+        for (int u = 0; u < 4; u++) k[u] = (i + u * kHistThreads < n) ? keys[i + u * kHistThreads] : 0;
 #pragma unroll
         for (int u = 0; u < 4; u++)
-            if (i + u * kSortThreads < n)
+            if (i + u * kHistThreads < n)
                 for (int p = 0; p < passes; p++) atomicAdd(&s_hist[p][(uint32_t)(k[u] >> plan.shift[p]) & ((1u << plan.bits[p]) - 1)], 1u);
     }
     __syncthreads();
     uint32_t *out = partials + (size_t)blockIdx.x * kMaxPasses * kRadix;
-    for (int p = 0; p < passes; p++) {
+    for (int j = tid; j < passes * kRadix; j += kHistThreads) {
         uint32_t sum = 0;
 #pragma unroll
-        for (int w = 0; w < kSortWaves; w++) sum += s_hist_wave[w][p][tid];
-        out[p * kRadix + tid] = sum;
+        for (int w = 0; w < kHistSets; w++) sum += s_hist_set[w][0][j];
+        out[j] = sum;
     }
 }
 
@@ -194,7 +196,7 @@ __device__ __forceinline__ void wave_match_rank_ballots(const uint32_t (&digit)[
 // One pass over digit (key >> shift) & mask, mask < 2^BITS.  `bases`: the exclusive scan of the digit totals,
 // or, with totals_given, the totals themselves (scanned here).
 template <int BITS>
-__global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t *__restrict__ keys_in,
+__global__ __launch_bounds__(kSweepThreads) void sort_sweep_kernel(const uint64_t *__restrict__ keys_in,
                                                                   const uint32_t *__restrict__ vals_in,
                                                                   uint64_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                                   int64_t n, int shift, uint32_t mask,
@@ -203,14 +205,16 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     constexpr int kDigits = 1 << BITS;
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_global_delta[kRadix];
-    __shared__ uint32_t s_scan_wave[kSortWaves];
-    __shared__ uint32_t s_base_wave[kSortWaves];
+    __shared__ uint32_t s_scan_wave[kSweepWaves];
+    __shared__ uint32_t s_base_wave[kSweepWaves];
     // The ranking counters are dead once every pair knows its place in the tile,
     // so they share LDS with the permutation buffer (51 KB: three workgroups per CU).
     __shared__ __align__(16) unsigned char s_raw[kSortTile * 12];
     uint32_t (*s_wave_count)[kRadix] = reinterpret_cast<uint32_t (*)[kRadix]>(s_raw);
-    uint32_t *s_local_start = reinterpret_cast<uint32_t *>(s_raw) + kSortWaves * kRadix;
-    unsigned long long *s_masks = reinterpret_cast<unsigned long long *>(s_raw + 8192);  // kSortWaves sets of kMaskWords
+    uint32_t *s_local_start = reinterpret_cast<uint32_t *>(s_raw) + kSweepWaves * kRadix;
+    constexpr int kMaskOffset = (kSweepWaves + 1) * kRadix * 4;
+    static_assert(kMaskOffset % 8 == 0 && kMaskOffset + kSweepWaves * kMaskWords * 8 <= kSortTile * 12, "counters and mask words fit the permutation buffer");
+    unsigned long long *s_masks = reinterpret_cast<unsigned long long *>(s_raw + kMaskOffset);  // kSweepWaves sets of kMaskWords
     uint64_t *s_keys = reinterpret_cast<uint64_t *>(s_raw);
     uint32_t *s_vals = reinterpret_cast<uint32_t *>(s_raw + kSortTile * 8);
 
@@ -219,8 +223,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const int wave = tid / kWave;
     const bool owns_digit = tid < kDigits;
     if (tid == 0) s_tile = ticket ? atomicAdd(ticket, 1u) : blockIdx.x;  // no ticket: the whole grid is resident
-    for (int w = 0; w < kSortWaves; w++) s_wave_count[w][tid] = 0;
-    for (int j = tid; j < kSortWaves * kMaskWords; j += kSortThreads) s_masks[j] = 0;
+    for (int j = tid; j < kSweepWaves * kRadix; j += kSweepThreads) s_wave_count[0][j] = 0;
+    for (int j = tid; j < kSweepWaves * kMaskWords; j += kSweepThreads) s_masks[j] = 0;
     // this digit's first output position: given, or the exclusive scan of the totals
     uint32_t base = owns_digit ? bases[totals_given ? tid * kTotalsStride : tid] : 0u;
     uint32_t base_incl = 0;
@@ -239,13 +243,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     const int n_valid = (int)((n - tile_base) < kSortTile ? (n - tile_base) : kSortTile);
 
     // Wave-striped loads keep memory order = (wave, item, lane) order.
-    uint64_t key[kSortItems];
-    uint32_t val[kSortItems];
-    uint32_t digit[kSortItems];
-    uint32_t rank[kSortItems];
-    const int lane_base = wave * (kWave * kSortItems) + lane;
+    uint64_t key[kSweepItems];
+    uint32_t val[kSweepItems];
+    uint32_t digit[kSweepItems];
+    uint32_t rank[kSweepItems];
+    const int lane_base = wave * (kWave * kSweepItems) + lane;
 #pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
+    for (int i = 0; i < kSweepItems; i++) {
         const int local = lane_base + i * kWave;
         if (local < n_valid) {
             key[i] = keys_in[tile_base + local];
@@ -256,16 +260,18 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         }
         digit[i] = (uint32_t)(key[i] >> shift) & mask;
     }
-    wave_match_rank<kSortItems>(digit, s_wave_count[wave], s_masks + wave * kMaskWords, rank);
+    wave_match_rank<kSweepItems>(digit, s_wave_count[wave], s_masks + wave * kMaskWords, rank);
     __syncthreads();
 
     // Thread d owns digit d: per-wave exclusive offsets, tile count, look-back.
     uint32_t digit_count = 0;
+    if (tid < kRadix) {
 #pragma unroll
-    for (int w = 0; w < kSortWaves; w++) {
-        const uint32_t c = s_wave_count[w][tid];
-        s_wave_count[w][tid] = digit_count;
-        digit_count += c;
+        for (int w = 0; w < kSweepWaves; w++) {
+            const uint32_t c = s_wave_count[w][tid];
+            s_wave_count[w][tid] = digit_count;
+            digit_count += c;
+        }
     }
     // real pairs only: padding always carries the largest digit
     const uint32_t published = ((uint32_t)tid == mask) ? digit_count - (uint32_t)(kSortTile - n_valid) : digit_count;
@@ -280,18 +286,18 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
         __syncthreads();
         uint32_t wave_prefix = 0;
         for (int w = 0; w < wave; w++) wave_prefix += s_scan_wave[w];
-        s_local_start[tid] = wave_prefix + v - digit_count;
+        if (tid < kRadix) s_local_start[tid] = wave_prefix + v - digit_count;
     }
 
     // Place of every pair inside the tile, then permute into digit order in LDS
     // (the buffer overlays the counters) and write digit runs contiguously.
-    const uint32_t local_start = s_local_start[tid];
     __syncthreads();  // s_local_start is complete
+    const uint32_t local_start = s_local_start[tid & (kRadix - 1)];
 #pragma unroll
-    for (int i = 0; i < kSortItems; i++) rank[i] += s_local_start[digit[i]] + s_wave_count[wave][digit[i]];
+    for (int i = 0; i < kSweepItems; i++) rank[i] += s_local_start[digit[i]] + s_wave_count[wave][digit[i]];
     __syncthreads();  // every pair knows its place: the counters may be overwritten
 #pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
+    for (int i = 0; i < kSweepItems; i++) {
         s_keys[rank[i]] = key[i];
         s_vals[rank[i]] = val[i];
     }
@@ -359,12 +365,12 @@ __global__ __launch_bounds__(kSortThreads) void sort_sweep_kernel(const uint64_t
     }
     const uint32_t prefix = group_prefix + in_group;
     if (timed_out && status) *status = TG_STATUS_LOOKBACK_TIMEOUT;
-    s_global_delta[tid] = base + prefix - local_start;
+    if (tid < kRadix) s_global_delta[tid] = base + prefix - local_start;
 
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < kSortItems; i++) {
-        const int pos = i * kSortThreads + tid;
+    for (int i = 0; i < kSweepItems; i++) {
+        const int pos = i * kSweepThreads + tid;
         if (pos < n_valid) {
             const uint64_t k = s_keys[pos];
             const uint32_t d = (uint32_t)(k >> shift) & mask;
@@ -574,29 +580,56 @@ __device__ __forceinline__ void segment_sort_in_wave(uint64_t *keys, uint32_t *v
     }
 }
 
-// One wave per segment; segments longer than kSegWaveCap are queued for segment_sort_large_kernel.
+// One workgroup per four segments.  A segment of up to kSegWaveCap pairs is sorted by one wave of its own;
+// then the workgroup takes those of up to kSegMediumCap pairs together, one after the other.  Longer ones are
+// left to segment_sort_large_kernel.
+constexpr int kSegMediumItems = 8;
+constexpr int kSegMediumCap = kSortThreads * kSegMediumItems;  // 2048 pairs: as much LDS as the four waves' own buffers
+struct MediumSegLds {
+    SegLds lds;
+    uint32_t ex_keys[kSegMediumCap], ex_vals[kSegMediumCap];
+};
 __global__ __launch_bounds__(kSortThreads) void segment_sort_small_kernel(uint64_t *keys, uint32_t *vals,
-                                                                          const int32_t *__restrict__ offsets, int n_segments,
-                                                                          uint32_t *queue_count, uint32_t *queue) {
-    __shared__ WaveSegLds lds_all[kSortWaves];
-    const int seg = blockIdx.x * kSortWaves + threadIdx.x / kWave;
-    if (seg >= n_segments) return;
-    WaveSegLds &lds = lds_all[threadIdx.x / kWave];
-    const int64_t start = offsets[seg];
-    const int n = offsets[seg + 1] - offsets[seg];
-    if (n <= 1) return;
-    if (n > kSegWaveCap) {
-        if ((threadIdx.x & (kWave - 1)) == 0) queue[atomicAdd(queue_count, 1u)] = (uint32_t)seg;
-        return;
+                                                                          const int32_t *__restrict__ offsets, int n_segments) {
+    __shared__ union SmallLds {
+        WaveSegLds wave[kSortWaves];
+        MediumSegLds medium;
+    } s;
+    const int wave = threadIdx.x / kWave;
+    const int first = blockIdx.x * kSortWaves;
+    int bounds[kSortWaves + 1];
+#pragma unroll
+    for (int w = 0; w <= kSortWaves; w++) bounds[w] = offsets[min(first + w, n_segments)];
+    bool any_medium = false;
+    int start = 0, n = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++) {
+        const int len = bounds[w + 1] - bounds[w];
+        any_medium = any_medium || (len > kSegWaveCap && len <= kSegMediumCap);
+        if (w == wave) { start = bounds[w]; n = len; }
     }
-    switch ((n + kWave - 1) / kWave) {
-    case 1: segment_sort_in_wave<1>(keys, vals, start, n, lds); break;
-    case 2: segment_sort_in_wave<2>(keys, vals, start, n, lds); break;
-    case 3: segment_sort_in_wave<3>(keys, vals, start, n, lds); break;
-    case 4: segment_sort_in_wave<4>(keys, vals, start, n, lds); break;
-    case 5: segment_sort_in_wave<5>(keys, vals, start, n, lds); break;
-    case 6: segment_sort_in_wave<6>(keys, vals, start, n, lds); break;
-    default: segment_sort_in_wave<8>(keys, vals, start, n, lds); break;
+    if (n > 1 && n <= kSegWaveCap) {
+        WaveSegLds &lds = s.wave[wave];
+        switch ((n + kWave - 1) / kWave) {
+        case 1: segment_sort_in_wave<1>(keys, vals, start, n, lds); break;
+        case 2: segment_sort_in_wave<2>(keys, vals, start, n, lds); break;
+        case 3: segment_sort_in_wave<3>(keys, vals, start, n, lds); break;
+        case 4: segment_sort_in_wave<4>(keys, vals, start, n, lds); break;
+        case 5: segment_sort_in_wave<5>(keys, vals, start, n, lds); break;
+        case 6: segment_sort_in_wave<6>(keys, vals, start, n, lds); break;
+        default: segment_sort_in_wave<8>(keys, vals, start, n, lds); break;
+        }
+    }
+    if (!any_medium) return;  // the same for the whole workgroup
+#pragma unroll 1
+    for (int w = 0; w < kSortWaves; w++) {
+        const int len = bounds[w + 1] - bounds[w];
+        if (len <= kSegWaveCap || len > kSegMediumCap) continue;
+        __syncthreads();  // the waves are done with their own buffers, the previous segment with the shared one
+        if (len <= kSortThreads * 4)
+            segment_sort_in_lds<4>(keys, vals, bounds[w], len, s.medium.lds, s.medium.ex_keys, s.medium.ex_vals);
+        else
+            segment_sort_in_lds<kSegMediumItems>(keys, vals, bounds[w], len, s.medium.lds, s.medium.ex_keys, s.medium.ex_vals);
     }
 }
 
@@ -682,21 +715,17 @@ __device__ void segment_sort_through_memory(uint64_t *keys, uint32_t *vals, uint
     }
 }
 
+// Segments longer than kSegMediumCap: the workgroups take them in turn.
 __global__ __launch_bounds__(kSortThreads, 2) void segment_sort_large_kernel(uint64_t *keys, uint32_t *vals, uint64_t *keys_alt,
-                                                                          uint32_t *vals_alt, const int32_t *__restrict__ offsets,
-                                                                          const uint32_t *queue_count, const uint32_t *queue) {
+                                                                             uint32_t *vals_alt, const int32_t *__restrict__ offsets,
+                                                                             int n_segments) {
     __shared__ SegLds lds;
     __shared__ uint32_t ex_keys[kSegLargeCap], ex_vals[kSegLargeCap];
-    const uint32_t queued = *queue_count;
-    for (uint32_t q = blockIdx.x; q < queued; q += gridDim.x) {
-        const int seg = (int)queue[q];
+    for (int seg = blockIdx.x; seg < n_segments; seg += gridDim.x) {
         const int64_t start = offsets[seg];
         const int n = offsets[seg + 1] - offsets[seg];
-        if (n <= kSortThreads * 4)
-            segment_sort_in_lds<4>(keys, vals, start, n, lds, ex_keys, ex_vals);
-        else if (n <= kSortThreads * 8)
-            segment_sort_in_lds<8>(keys, vals, start, n, lds, ex_keys, ex_vals);
-        else if (n <= kSortThreads * 16)
+        if (n <= kSegMediumCap) continue;
+        if (n <= kSortThreads * 16)
             segment_sort_in_lds<16>(keys, vals, start, n, lds, ex_keys, ex_vals);
         else if (n <= kSegLargeCap)
             segment_sort_in_lds<kSegLargeItems>(keys, vals, start, n, lds, ex_keys, ex_vals);
@@ -719,7 +748,7 @@ template <int BITS>
 static void launch_sweep(dim3 grid, hipStream_t s, const uint64_t *kin, const uint32_t *vin, uint64_t *kout, uint32_t *vout,
                          int64_t n, int shift, uint32_t mask, const uint32_t *bases, int totals_given, uint32_t *lookback,
                          uint32_t *ticket, uint32_t *status) {
-    hipLaunchKernelGGL(sort_sweep_kernel<BITS>, grid, dim3(kSortThreads), 0, s, kin, vin, kout, vout, n, shift, mask, bases,
+    hipLaunchKernelGGL(sort_sweep_kernel<BITS>, grid, dim3(kSweepThreads), 0, s, kin, vin, kout, vout, n, shift, mask, bases,
                        totals_given, lookback, ticket, status);
 }
 
@@ -734,7 +763,7 @@ static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, co
     // 534 same-address ticket atomics cost 6 us per pass; a grid that fits the device whole takes its
     // tile numbers from the workgroup ids instead
     static int resident_cache[kMaxDevices] = {0};
-    const bool whole_grid_resident = n_sort_tiles <= resident_workgroups((const void *)sort_sweep_kernel<kRadixBits>, kSortThreads, resident_cache);
+    const bool whole_grid_resident = n_sort_tiles <= resident_workgroups((const void *)sort_sweep_kernel<kRadixBits>, kSweepThreads, resident_cache);
     // one pair of timing events around all passes: a pair per launch would add its own two
     // microseconds to every 24 us kernel
     ProfileScope timed("sort_sweep_kernel", s, plan.passes);
@@ -766,7 +795,7 @@ static int run_passes(const char *fn, const PassPlan &plan, const SortLayout &L,
     uint32_t *partials = (uint32_t *)(ws + L.off_partials);
     uint32_t *lookback = (uint32_t *)(ws + L.off_lookback);
     // tickets and look-back words (adjacent) start at zero; bases and partials are fully overwritten
-    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kSortThreads), 0, s, keys, n, plan, partials, tickets, L.zero_words);
+    TG_LAUNCH(sort_histogram_kernel, dim3(L.hist_blocks), dim3(kHistThreads), 0, s, keys, n, plan, partials, tickets, L.zero_words);
     if (int e = check_launch("sort_histogram_kernel")) return e;
     TG_LAUNCH(sort_bases_kernel, dim3(plan.passes), dim3(kBasesThreads), 0, s, partials, L.hist_blocks, bases, status);
     if (int e = check_launch("sort_bases_kernel")) return e;
@@ -775,14 +804,13 @@ static int run_passes(const char *fn, const PassPlan &plan, const SortLayout &L,
 
 // Tile ranges of keys that are ordered by tile, then every tile's segment sorted by its depth bits in place.
 static int ranges_and_segments(uint64_t *k, uint32_t *v, uint64_t *k_other, uint32_t *v_other, int64_t n, int n_tiles,
-                               int32_t *offsets, uint32_t *queue_count, uint32_t *queue, hipStream_t s) {
+                               int32_t *offsets, hipStream_t s) {
     TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n + 1, kSortThreads)), dim3(kSortThreads), 0, s, k, n, n_tiles, offsets);
     if (int e = check_launch("tile_ranges_kernel")) return e;
-    TG_LAUNCH(segment_sort_small_kernel, dim3(ceil_div(n_tiles, kSortWaves)), dim3(kSortThreads), 0, s, k, v, offsets, n_tiles,
-              queue_count, queue);
+    TG_LAUNCH(segment_sort_small_kernel, dim3(ceil_div(n_tiles, kSortWaves)), dim3(kSortThreads), 0, s, k, v, offsets, n_tiles);
     if (int e = check_launch("segment_sort_small_kernel")) return e;
-    TG_LAUNCH(segment_sort_large_kernel, dim3(kSegLargeGrid), dim3(kSortThreads), 0, s, k, v, k_other, v_other, offsets,
-              queue_count, queue);
+    TG_LAUNCH(segment_sort_large_kernel, dim3(n_tiles < kSegLargeGrid ? n_tiles : kSegLargeGrid), dim3(kSortThreads), 0, s, k, v,
+              k_other, v_other, offsets, n_tiles);
     return check_launch("segment_sort_large_kernel");
 }
 
@@ -805,7 +833,7 @@ using namespace tg;
 
 extern "C" size_t tg_sort_workspace_bytes(int64_t n) {
     if (n < 0 || n > kSortMaxN) return 0;
-    return sort_layout(n, kMaxPasses, 0).total;
+    return sort_layout(n, kMaxPasses).total;
 }
 
 extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
@@ -826,7 +854,7 @@ extern "C" int tg_sort_pairs_u64_u32(uint64_t *keys, uint32_t *values, uint64_t 
     }
     if (int e = check_sort_buffers("tg_sort_pairs_u64_u32", keys, values, keys_alt, values_alt, workspace)) return e;
     const PassPlan plan = plan_passes(0, end_bit);
-    const SortLayout L = sort_layout(n, plan.passes, 0);
+    const SortLayout L = sort_layout(n, plan.passes);
     if (workspace_bytes < L.total) {
         set_error("tg_sort_pairs_u64_u32: workspace of %zu bytes, need %zu", workspace_bytes, L.total);
         return TG_E_WORKSPACE;
@@ -849,7 +877,7 @@ extern "C" int tg_tile_ranges(const uint64_t *sorted_keys, int64_t n_keys, int n
 
 extern "C" size_t tg_tile_list_sort_workspace_bytes(int64_t n, int n_tiles) {
     if (n < 0 || n > kSortMaxN || n_tiles <= 0) return 0;
-    return sort_layout(n, kMaxPasses / 2, n_tiles).total;
+    return sort_layout(n, kMaxPasses / 2).total;
 }
 
 // (keys, values): n > 0 pairs in any order -> tile passes with a histogram of their own, ranges, segments.
@@ -858,7 +886,7 @@ static int sort_tile_lists_run(const char *fn, uint64_t *keys, uint32_t *values,
                                int *result_in_alt, hipStream_t s) {
     if (int e = check_sort_buffers(fn, keys, values, keys_alt, values_alt, workspace)) return e;
     const PassPlan plan = tile_pass_plan(n_tiles);
-    const SortLayout L = sort_layout(n, plan.passes, n_tiles);
+    const SortLayout L = sort_layout(n, plan.passes);
     if (workspace_bytes < L.total) {
         set_error("%s: workspace of %zu bytes, need %zu", fn, workspace_bytes, L.total);
         return TG_E_WORKSPACE;
@@ -868,8 +896,7 @@ static int sort_tile_lists_run(const char *fn, uint64_t *keys, uint32_t *values,
     uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
     uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
     *result_in_alt = (plan.passes & 1);
-    return ranges_and_segments(k, v, k_other, v_other, n, n_tiles, offsets, (uint32_t *)(ws + L.off_tickets) + kQueueCountWord,
-                               (uint32_t *)(ws + L.off_queue), s);
+    return ranges_and_segments(k, v, k_other, v_other, n, n_tiles, offsets, s);
 }
 
 extern "C" int tg_sort_tile_lists(uint64_t *keys, uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int64_t n,
@@ -909,7 +936,7 @@ constexpr int kEmitDigitPasses = 2;
 extern "C" size_t tg_build_tile_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
     if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0) return 0;
     if (tile_pass_plan(n_tiles).passes > kEmitDigitPasses) return tg_tile_list_sort_workspace_bytes(n_keys, n_tiles);
-    return build_lookback_bytes(n_keys, n_tiles) + (size_t)n_tiles * 4;
+    return build_lookback_bytes(n_keys, n_tiles);
 }
 
 extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
@@ -954,12 +981,11 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     }
     if (int e = check_sort_buffers("tg_build_tile_lists", keys, values, keys_alt, values_alt, workspace)) return e;
     const size_t lookback_bytes = build_lookback_bytes(n_keys, n_tiles);
-    if (workspace_bytes < lookback_bytes + (size_t)n_tiles * 4) {
-        set_error("tg_build_tile_lists: workspace of %zu bytes, need %zu", workspace_bytes, lookback_bytes + (size_t)n_tiles * 4);
+    if (workspace_bytes < lookback_bytes) {
+        set_error("tg_build_tile_lists: workspace of %zu bytes, need %zu", workspace_bytes, lookback_bytes);
         return TG_E_WORKSPACE;
     }
     uint32_t *lookback = (uint32_t *)workspace;
-    uint32_t *queue = (uint32_t *)((char *)workspace + lookback_bytes);
     // the emission clears the look-back words and the status word; the digit totals are the binning kernel's
     if (int e = launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads, frame,
                                     width, height, tile_w, tile_h, keys, values, lookback, lookback_bytes / 4, status, s))
@@ -973,5 +999,5 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
     uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
     *result_in_alt = (plan.passes & 1);
-    return ranges_and_segments(k, v, k_other, v_other, n_keys, n_tiles, offsets, tickets + kQueueCountWord, queue, s);
+    return ranges_and_segments(k, v, k_other, v_other, n_keys, n_tiles, offsets, s);
 }

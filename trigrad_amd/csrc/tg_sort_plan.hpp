@@ -12,6 +12,12 @@ constexpr int kSortThreads = 256;
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kSortItems = 16;
 constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
+#ifndef TG_SWEEP_THREADS
+#define TG_SWEEP_THREADS 512
+#endif
+constexpr int kSweepThreads = TG_SWEEP_THREADS;  // the sweep spreads a tile over more waves than it has digits to own
+constexpr int kSweepWaves = kSweepThreads / kWave;
+constexpr int kSweepItems = kSortTile / kSweepThreads;
 constexpr int kHistBlocksMax = 256;
 constexpr int kBasesThreads = 1024;
 constexpr int kLookWindow = 8;  // look-back words a digit's thread reads per round trip
@@ -52,27 +58,24 @@ inline size_t lookback_words_per_pass(int64_t n_sort_tiles) {
 struct SortLayout {
     int n_tiles;
     int hist_blocks;
-    size_t off_tickets, off_partials, off_bases, off_lookback, off_queue, total;
+    size_t off_tickets, off_partials, off_bases, off_lookback, total;
     size_t zero_words;  // words from off_tickets on that must be zero before the sweeps start
 };
 
-// queue_entries: room for that many segment numbers behind the look-back words (tile list sort only)
-inline SortLayout sort_layout(int64_t n, int passes, int64_t queue_entries) {
+inline SortLayout sort_layout(int64_t n, int passes) {
     SortLayout L;
     L.n_tiles = (int)ceil_div64(n, kSortTile);
     L.hist_blocks = L.n_tiles < kHistBlocksMax ? (L.n_tiles > 0 ? L.n_tiles : 1) : kHistBlocksMax;
     size_t o = 0;
     L.off_bases = o;    o += (size_t)kMaxPasses * kRadix * 4;
     L.off_partials = o; o += (size_t)kHistBlocksMax * kMaxPasses * kRadix * 4;
-    L.off_tickets = o;  o += 256;  // kMaxPasses tickets, the status of the segment kernels, the queue length; zeroed with the look-back words
+    L.off_tickets = o;  o += 256;  // kMaxPasses tickets; zeroed with the look-back words
     L.off_lookback = o; o += (size_t)passes * lookback_words_per_pass(L.n_tiles > 0 ? L.n_tiles : 1) * 4;
     L.zero_words = (o - L.off_tickets) / 4;
-    L.off_queue = o;    o += (size_t)queue_entries * 4;
     L.total = o;
     return L;
 }
 constexpr int kTotalsStride = 1;  // words between two digit totals (a cache line each was tried: the atomics got no faster)
-constexpr int kQueueCountWord = 32;  // word of the ticket block that counts the queued segments
 
 
 // Key bits that hold a tile number below n_tiles (at least one).
