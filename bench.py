@@ -31,9 +31,10 @@ sys.path.insert(1, os.path.join(ROOT, "tests"))  # the seeded scene generators l
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of sort_sweep_kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
-# 256 MiB plain copy (profiles/config2_hbm_traffic_counters.md), keyed by the number of pairs it was measured on.
-MEASURED_SWEEP_TRAFFIC = {2186877: 64.2e6}
+# Bytes per launch of sort_sweep_kernel that pass the L2 on their way to the fabric, measured with rocprofv3 --pmc: read and
+# write requests by size (and, agreeing within 0.2 %, FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB plain copy), keyed by
+# the number of pairs it was measured on (profiles/config2_hbm_traffic_counters.md).
+MEASURED_SWEEP_TRAFFIC = {2186877: 57.0e6}
 
 MODES = {
     "A": dict(per_pixel_sort=True, max_layers=32),    # API defaults
