@@ -5,7 +5,9 @@
  *   - every pointer is a DEVICE pointer unless its comment says "host";
  *   - the library allocates nothing and keeps no state between calls: the
  *     caller owns every buffer, including workspaces, whose size the
- *     *_workspace_bytes functions report;
+ *     *_workspace_bytes functions report (one entry point,
+ *     tg_scan_exclusive_u32_noalloc, works in a device array of its own
+ *     instead of a workspace);
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all
  *     work is enqueued on it and no entry point synchronises;
  *   - the return value is 0 on success, a negative TG_E_* code for rejected
@@ -46,7 +48,14 @@ typedef float tg_real;
 
 #define TG_MAX_SAVED_LAYERS 32 /* largest max_layers for which the forward pass can save the blend order */
 
-/* Status word values written by the kernels that wait on other workgroups. */
+/* Status word values written by the kernels that wait on other workgroups
+ * (the scans' and the sweeps' decoupled look-back).  Their waits are bounded: a
+ * wait that expires sets TG_STATUS_LOOKBACK_TIMEOUT and the kernel carries on,
+ * so every wave exits; the results of that call are then invalid and the
+ * caller must look at the word before it trusts them.  A grid that fits the
+ * device whole numbers its tiles by workgroup id (every workgroup it waits
+ * for is resident by then); that presumes the kernel has the device to itself.
+ * With other streams or processes on the GPU a wait can expire. */
 #define TG_STATUS_OK 0u
 #define TG_STATUS_LOOKBACK_TIMEOUT 1u
 
