@@ -58,6 +58,20 @@ def test_host_side_helpers_and_argument_rejection(bits):
     assert lib.tg_hit_mask_words(6400, 64, 64, 16, 16) == 16 + (100 + 16 + 1) * 256  # a word per workgroup, then the chunks
     assert lib.tg_list_bound_words(6400, 16) == 25 + 16 + 1
     assert lib.tg_list_bounds(None, 0, None, 0, None, None, None, 0, None, None, None, None) == -1
+    # the frame's two calls and the tile-list sort
+    assert lib.tg_bin_setup_workspace_bytes(10 ** 6, 1920, 1080, 16, 16) % 256 == 0
+    assert 0 < lib.tg_bin_setup_workspace_bytes(0, 64, 64, 16, 16) < 10 ** 4
+    assert lib.tg_bin_setup_workspace_bytes(-1, 64, 64, 16, 16) == 0
+    assert lib.tg_bin_setup(None, 0, None, 5, 64, 64, 16, 16, None, None, None, 0, None, None, 0, None) == -1
+    assert b"tg_bin_setup" in lib.tg_last_error()
+    assert lib.tg_build_tile_lists_workspace_bytes(10 ** 6, 8160) > 0 and lib.tg_build_tile_lists_workspace_bytes(1 << 30, 8160) == 0
+    assert lib.tg_tile_list_sort_workspace_bytes(10 ** 6, 0) == 0
+    res = C.c_int(7)
+    assert lib.tg_build_tile_lists(None, None, 5, 10, 0, None, None, 64, 64, 16, 16, None, None, None, None, None, None, 0, None, 0,
+                                   C.byref(res), None) == -1
+    assert lib.tg_sort_tile_lists(None, None, None, None, 10, 0, None, None, 0, None, C.byref(res), None) == -1
+    assert lib.tg_scan_noalloc_max_n() == 1 << 24
+    assert lib.tg_scan_exclusive_u32_noalloc(None, None, (1 << 24) + 1, None, None, 256, 0, None, None) == -1
     with pytest.raises(RuntimeError, match="tg_bin_count failed with code -1"):
         _lib.check(lib.tg_bin_count(None, 0, None, -1, 64, 64, 16, 16, None, None), "tg_bin_count", bits)
 

@@ -159,6 +159,13 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
         if (!__syncthreads_or(want)) break;
         const int cap = want ? min(kLayers, a.max_layers - s.blended) : 0;
         int found = 0;
+        // The records of the next batch are fetched into registers while this batch is worked on: the
+        // chain of dependent loads (list -> indices -> vertices, matrix) of a batch takes as long as its
+        // inside tests, and with two workgroups per CU nothing else would cover it.  (Not with depth
+        // bounds, which make the batches jump.)
+        const bool ahead = !a.batch_bounds && (int)blockDim.x >= kStage;
+        DepthRecord fetched;
+        if (ahead && tid < min(kStage, end - start)) gather_depth(a, start + tid, fetched);
         for (int batch = start; batch < end; batch += kStage) {
             const int nb = min(kStage, end - batch);
             if (a.batch_bounds) {
@@ -176,11 +183,19 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 }
             }
             __syncthreads();
-            for (int e = tid; e < nb; e += blockDim.x) {
-                gather_depth(a, batch + e, s_rec[e]);
-                s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+            if (ahead) {
+                if (tid < nb) {
+                    s_rec[tid] = fetched;
+                    s_touch[tid] = (uint8_t)waves_touched(fetched.m, s_rects, n_waves);
+                }
+            } else {
+                for (int e = tid; e < nb; e += blockDim.x) {
+                    gather_depth(a, batch + e, s_rec[e]);
+                    s_touch[e] = (uint8_t)waves_touched(s_rec[e].m, s_rects, n_waves);
+                }
             }
             __syncthreads();
+            if (ahead && batch + kStage < end && tid < min(kStage, end - batch - kStage)) gather_depth(a, batch + kStage + tid, fetched);
             // inside tests into a per-lane mask, then every lane visits its own hits in
             // list order (the order insert_sorted_topk sees them in the reference)
             uint64_t m[kStage / kWave];

@@ -10,7 +10,10 @@ constexpr int kRadix = 1 << kRadixBits;
 constexpr int kMaxPasses = 8;
 constexpr int kSortThreads = 256;
 constexpr int kSortWaves = kSortThreads / kWave;
-constexpr int kSortItems = 16;
+#ifndef TG_SORT_ITEMS
+#define TG_SORT_ITEMS 16
+#endif
+constexpr int kSortItems = TG_SORT_ITEMS;
 constexpr int kSortTile = kSortThreads * kSortItems;  // 4096 pairs
 #ifndef TG_SWEEP_THREADS
 #define TG_SWEEP_THREADS 512
