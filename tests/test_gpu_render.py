@@ -88,6 +88,44 @@ def test_forward_matches_oracle(name, mode, cuda, oracle):
     _check_forward(f"{name}/{mode}", want, got)
 
 
+def _long_list_scene():
+    """One 16x16 tile whose list is longer than 65535 entries next to tiles with short lists: the per-pixel-order
+    forward pass keeps list positions in 16 bits where they fit and hands the other tiles to a second launch."""
+    import scenes as S
+    crowd = S.random_soup(70000, 32, 32, seed=3, sigma_px=1.5, opacity=(0.02, 0.2))
+    v = crowd["vertices"].copy()
+    v[:, :2] = v[:, :2] * 0.45 - 0.5  # into the first tile (with a fringe over its neighbours)
+    rest = S.random_soup(1500, 32, 32, seed=4, sigma_px=5.0)
+    vertices = np.concatenate([v, rest["vertices"]])
+    indices = np.concatenate([crowd["indices"], rest["indices"] + v.shape[0]]).astype(np.int32)
+    scene = dict(crowd)
+    scene.update(vertices=vertices, indices=indices, colors=np.concatenate([crowd["colors"], rest["colors"]]),
+                 opacities=np.concatenate([crowd["opacities"], rest["opacities"]]))
+    return scene
+
+
+@pytest.mark.parametrize("mode", ["A_default", "A_40_layers", "B_3_layers"])
+def test_tile_list_longer_than_16_bit_positions(mode, cuda, oracle):
+    import torch
+    from trigrad_amd import _C
+    scene = _long_list_scene()
+    m = MODES[mode]
+    d, want, got, ml = _forward_both(scene, 16, 16, m, cuda, oracle)
+    lengths = np.diff(want["offsets"])
+    assert lengths.max() > 65535 and lengths.min() < 65535
+    _check_forward(f"long list/{mode}", want, got)
+    gi, gd = _grad_inputs(scene, 9, True)
+    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                        32, 32, 16, 16, m["per_pixel_sort"], ml, literal=False)
+    image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
+    out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
+                             d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, 32, 32,
+                             16, 16, 1 / 256, m["per_pixel_sort"], ml, resume=resume)
+    for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
+        scale = float(np.abs(w).max())
+        assert_close(f"long list/{mode}: {label}", g.cpu().numpy().astype(np.float64), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * scale)
+
+
 def _grad_inputs(scene, seed, with_depth):
     rng = np.random.default_rng(seed)
     H, W = scene["height"], scene["width"]

@@ -783,22 +783,34 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 }
 
 // Per-pixel order with the blend order saved by the forward pass
-// (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  Every wave walks its 64
-// pixels in lockstep, each lane from its own far end; a lane gathers the record of
-// its fragment from memory (neighbouring pixels hold the same few entries, so the
-// loads hit in cache; staging the tile's records in LDS first was measured slower,
-// for the workgroups per CU it costs).  LDS floating-point atomics cost about three
-// cycles per lane on gfx950 and many lanes of a wave hold the same entry in the same
-// step, so the 21 gradient terms of a step are grouped by entry first: lanes with
-// equal entries get consecutive slots (ballot matching, groups in order of their
-// lowest lane), the terms go to a slot-major matrix in LDS, three groups of 21 lanes
-// add up the runs of equal entry and issue one global floating-point atomic per run
-// and term.
+// (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  Step s of a pixel is its
+// fragment n - 1 - s, so every pixel starts at its own far end.  The pixels of a wave
+// hold different numbers of fragments, so the (pixel, step) pairs of the wave are
+// numbered step by step, the pixels that still have a fragment in lane order inside a
+// step, and taken 64 at a time: a round's 64 slots keep every lane busy whatever
+// the pixels' counts are, and a pixel's own slots come in the order it must visit
+// them.  Per round:
+//   1. lane = pixel: which of my steps own a slot of the round; their list positions
+//      (fetched from the saved order a few steps ahead) go to the slots;
+//   2. lane = slot: gathers the record of its fragment from memory (neighbouring
+//      pixels hold the same few entries, so the loads hit in cache; staging the tile's
+//      records in LDS first was measured slower, for the workgroups per CU it costs)
+//      and leaves the fragment's own opacity, colour and view depth in the slot;
+//   3. lane = pixel: the ordered part over my slots of the round, which replaces the
+//      five values by the five numbers the gradient terms are linear in;
+//   4. lane = slot: the 21 gradient terms.  LDS floating-point atomics cost about three
+//      cycles per lane on gfx950 and many slots of a round hold the same entry, so the
+//      terms are grouped by entry first: slots with equal entries get consecutive
+//      columns (ballot matching, groups in order of their lowest slot) of a term
+//      matrix in LDS, three groups of 21 lanes add up the runs of equal entry and issue
+//      one global floating-point atomic per run and term.
 template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ real s_term[kMaxWaves][kTerms * kTermStride];
-    __shared__ int s_tag[kMaxWaves][kWave];
-    __shared__ int s_vertex[kMaxWaves][3 * kWave];  // the three vertex ids of a slot's entry
+    __shared__ int s_rel[kMaxWaves][kWave];         // list position of a slot's fragment, from the tile's start
+    __shared__ int s_tag[kMaxWaves][kWave];         // the same by column of the term matrix
+    __shared__ int s_vertex[kMaxWaves][3 * kWave];  // the three vertex ids of a column's entry
+    __shared__ uint8_t s_src[kMaxWaves][kWave];     // the pixel (lane) of a slot
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
@@ -807,8 +819,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     const PixelCoord p = pixel_of_thread(a);
     const int rel_bits = 32 - __builtin_clz(max(end - start - 1, 1));  // bits that tell two list positions apart
     real *terms = s_term[wave];
+    int *rels = s_rel[wave];
     int *tags = s_tag[wave];
     int *vertices = s_vertex[wave];
+    uint8_t *srcs = s_src[wave];
     const TermLane tl = term_lane<kLayout>(g, lane);
 
     BackState st;
@@ -817,55 +831,115 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
         st = load_back_state(g, p);
         n = min(g.ends[p.index], a.max_layers);  // render.cu:642
     }
-    int n_max = n;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) n_max = max(n_max, __shfl_xor(n_max, off, kWave));
     const int64_t plane = (int64_t)a.W * a.H;
-    // step s of a lane is its layer n - 1 - s: every lane starts at its own far end
-    for (int s0 = 0; s0 < n_max; s0 += kGatherAhead) {
-        int rel[kGatherAhead];
-#pragma unroll
-        for (int u = 0; u < kGatherAhead; u++)
-            rel[u] = (n > 0) ? g.fragments[(int64_t)max(n - 1 - s0 - u, 0) * plane + p.index] : 0;
-#pragma unroll
-        for (int u = 0; u < kGatherAhead; u++) {
-            if (s0 + u >= n_max) break;  // wave-uniform
-            const bool active = s0 + u < n;
-            real term[kTerms];
-            BackRecord r;
-            if (active) {
-                gather_back(a, start + rel[u], r);
-                real b0, b1, b2;
-                bary_apply(r.m, p.px, p.py, b0, b1, b2);
-                fragment_backward(st, r, b0, b1, b2, p.px, p.py, term);
+    auto position_of_step = [&](int s) { return (s < n) ? g.fragments[(int64_t)(n - 1 - s) * plane + p.index] : 0; };
+    // the list positions of my next four steps
+    int ahead0 = position_of_step(0), ahead1 = position_of_step(1), ahead2 = position_of_step(2), ahead3 = position_of_step(3);
+    const int total = __builtin_amdgcn_readlane((int)wave_inclusive_scan_u32((uint32_t)n), kWave - 1);
+
+    int step = 0, step_base = 0;  // wave-uniform: the first step with a slot left, and the number of its first slot
+    for (int round0 = 0; round0 < total; round0 += kWave) {
+        const int n_slots = min(kWave, total - round0);
+        // 1. the round's slots
+        uint64_t mine = 0;  // my slots of the round: increasing slot = increasing step
+        while (step_base < round0 + kWave) {
+            const uint64_t votes = __builtin_amdgcn_ballot_w64(n > step);
+            if (votes == 0) break;
+            const int count = __builtin_popcountll(votes);
+            const int slot = step_base + (int)lanes_below_mask(votes) - round0;
+            if (n > step && slot >= 0 && slot < kWave) {
+                mine |= 1ull << slot;
+                rels[slot] = ahead0;
+                srcs[slot] = (uint8_t)lane;
+                ahead0 = ahead1; ahead1 = ahead2; ahead2 = ahead3;
+                ahead3 = position_of_step(step + 4);
             }
-            // slots: lanes with the same entry next to each other, groups in order of their lowest lane
-            uint64_t peers = __builtin_amdgcn_ballot_w64(active);
-            for (int b = 0; b < rel_bits; b++) {  // wave-uniform
-                const bool bit = (rel[u] >> b) & 1;
-                const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
-                peers &= bit ? vote : ~vote;
-            }
-            const uint32_t rank = lanes_below_mask(peers);
-            const bool leads = active && rank == 0;
-            const uint32_t size = leads ? (uint32_t)__builtin_popcountll(peers) : 0u;
-            const uint32_t incl = wave_inclusive_scan_u32(size);
-            const int n_slots = __builtin_amdgcn_readlane((int)incl, kWave - 1);
-            const int leader = active ? __builtin_ctzll(peers) : lane;
-            const int slot = __shfl((int)(incl - size), leader, kWave) + (int)rank;
-            if (active) {
-#pragma unroll
-                for (int q = 0; q < kTerms; q++) terms[q * kTermStride + slot] = term[q];
-                tags[slot] = rel[u];
-#pragma unroll
-                for (int k = 0; k < 3; k++) vertices[k * kWave + slot] = r.id[k];
-            }
-            wave_lds_sync();
-            // a slot starts a run where its entry differs from the slot before
-            const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tags[lane] != tags[max(lane - 1, 0)]));
-            add_run_sums(terms, n_slots, heads, tl, [&](int c, int v) { return vertices[v * kWave + c]; });
-            wave_lds_sync();
+            if (step_base + count > round0 + kWave) break;  // the step goes on in the next round
+            step_base += count;
+            step++;
         }
+        wave_lds_sync();
+
+        // 2. lane = slot: the record, and the fragment's own values
+        const int src = (lane < n_slots) ? srcs[lane] : lane;
+        const real px = __shfl(p.px, src, kWave), py = __shfl(p.py, src, kWave);
+        BackRecord r;
+        real b0 = 0.0f, b1 = 0.0f, b2 = 0.0f;
+        int rel = 0;
+        if (lane < n_slots) {
+            rel = rels[lane];
+            gather_back(a, start + rel, r);
+            bary_apply(r.m, px, py, b0, b1, b2);
+            const FragValue v = fragment_value(r, b0, b1, b2);
+            terms[0 * kTermStride + lane] = v.o;
+            terms[1 * kTermStride + lane] = v.color[0];
+            terms[2 * kTermStride + lane] = v.color[1];
+            terms[3 * kTermStride + lane] = v.color[2];
+            terms[4 * kTermStride + lane] = v.z;
+        }
+        wave_lds_sync();
+
+        // 3. lane = pixel: the ordered part
+        while (true) {
+            const bool active = mine != 0;
+            if (__builtin_amdgcn_ballot_w64(active) == 0) break;
+            if (active) {
+                const int c = __builtin_ctzll(mine);
+                mine &= mine - 1;
+                FragValue v;
+                v.o = terms[0 * kTermStride + c];
+                v.color[0] = terms[1 * kTermStride + c];
+                v.color[1] = terms[2 * kTermStride + c];
+                v.color[2] = terms[3 * kTermStride + c];
+                v.z = terms[4 * kTermStride + c];
+                const FragSeed f = fragment_chain_step(st, v);
+                terms[0 * kTermStride + c] = f.d_do;
+                terms[1 * kTermStride + c] = f.gc[0];
+                terms[2 * kTermStride + c] = f.gc[1];
+                terms[3 * kTermStride + c] = f.gc[2];
+                terms[4 * kTermStride + c] = f.dd_dz;
+            }
+        }
+        wave_lds_sync();
+
+        // 4. lane = slot: the terms, in the column the matching gives the slot
+        const bool active = lane < n_slots;
+        FragSeed f;
+        f.d_do = f.gc[0] = f.gc[1] = f.gc[2] = f.dd_dz = 0.0f;
+        if (active) {
+            f.d_do = terms[0 * kTermStride + lane];
+            f.gc[0] = terms[1 * kTermStride + lane];
+            f.gc[1] = terms[2 * kTermStride + lane];
+            f.gc[2] = terms[3 * kTermStride + lane];
+            f.dd_dz = terms[4 * kTermStride + lane];
+        }
+        uint64_t peers = __builtin_amdgcn_ballot_w64(active);
+        for (int b = 0; b < rel_bits; b++) {  // wave-uniform
+            const bool bit = (rel >> b) & 1;
+            const uint64_t vote = __builtin_amdgcn_ballot_w64(bit);
+            peers &= bit ? vote : ~vote;
+        }
+        const uint32_t rank = lanes_below_mask(peers);
+        const bool leads = active && rank == 0;
+        const uint32_t size = leads ? (uint32_t)__builtin_popcountll(peers) : 0u;
+        const uint32_t incl = wave_inclusive_scan_u32(size);
+        const int leader = active ? __builtin_ctzll(peers) : lane;
+        const int column = __shfl((int)(incl - size), leader, kWave) + (int)rank;
+        wave_lds_sync();  // every slot's five numbers are in registers before terms take their place
+        if (active) {
+            real term[kTerms];
+            fragment_terms(f, r, b0, b1, b2, px, py, term);
+#pragma unroll
+            for (int q = 0; q < kTerms; q++) terms[q * kTermStride + column] = term[q];
+            tags[column] = rel;
+#pragma unroll
+            for (int k = 0; k < 3; k++) vertices[k * kWave + column] = r.id[k];
+        }
+        wave_lds_sync();
+        // a column starts a run where its entry differs from the column before
+        const uint64_t heads = __builtin_amdgcn_ballot_w64(lane < n_slots && (lane == 0 || tags[lane] != tags[max(lane - 1, 0)]));
+        add_run_sums(terms, n_slots, heads, tl, [&](int c, int v) { return vertices[v * kWave + c]; });
+        wave_lds_sync();
     }
 }
 

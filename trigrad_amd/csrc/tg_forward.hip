@@ -115,7 +115,8 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
 }
 
 // render.cu:338-373 insert_sorted_topk on an LDS candidate list of capacity `cap`.
-__device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, real d, int j) {
+template <typename Pos>
+__device__ __forceinline__ void topk_insert(const TopKOf<Pos> &tk, int cap, int &n, real d, int j) {
     if (n == cap && d >= tk.d(cap - 1)) return;
     int i = (n < cap) ? n : cap - 1;
     while (i > 0 && d < tk.d(i - 1)) {
@@ -124,35 +125,39 @@ __device__ __forceinline__ void topk_insert(const TopK &tk, int cap, int &n, rea
         i--;
     }
     tk.d(i) = d;
-    tk.j(i) = j;
+    tk.j(i) = (Pos)j;
     if (n < cap) n++;
 }
 
-constexpr int kSelectBatch = 128;
+constexpr int kSelectBatch = 128;       // list entries staged per batch where positions take an int
+constexpr int kSelectBatchShort = 64;   // ... and where they take 16 bits
+constexpr int kShortList = 0xffff;      // longest tile list whose positions fit 16 bits
+constexpr int kLongListGroups = 256;    // workgroups that look for the tiles with longer lists
 
-template <int kStage>  // list entries staged per batch
-__global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(RasterArgs a, ForwardOut out) {
-    extern __shared__ __align__(16) unsigned char s_dyn[];
+// The per-pixel-order forward pass of one tile.  Pos: how a candidate's list position (from the tile's
+// start) is kept.  With uint16_t the candidate lists of a 16x16 tile take 48 KB instead of 64 KB, which
+// together with 64 staged entries lets a CU hold three workgroups instead of two.
+template <int kStage, typename Pos>  // kStage: list entries staged per batch
+__device__ __forceinline__ void pixel_order_tile(const RasterArgs &a, const ForwardOut &out, int tile_x, int tile_y, int tiles_x,
+                                                 unsigned char *s_dyn, uint8_t *s_touch, WaveRect *s_rects) {
     const int n_threads = blockDim.x;
     DepthRecord *s_rec = reinterpret_cast<DepthRecord *>(s_dyn);
-    TopK tk;
+    TopKOf<Pos> tk;
     tk.depth = reinterpret_cast<real *>(s_dyn + sizeof(DepthRecord) * kStage);
-    tk.pos = reinterpret_cast<int *>(tk.depth + kLayers * n_threads);
+    tk.pos = reinterpret_cast<Pos *>(tk.depth + kLayers * n_threads);
     tk.n_threads = n_threads;
 
-    __shared__ uint8_t s_touch[kStage];
-    __shared__ WaveRect s_rects[kMaxTileWaves];
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
     const int n_waves = blockDim.x / kWave;
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = tile_y * tiles_x + tile_x;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
-    const PixelCoord p = pixel_of_thread(a);
+    const PixelCoord p = pixel_of_thread(a, tile_x, tile_y);
     publish_wave_rect(p, s_rects);
 
     PixelState s;
     real last_depth = -__builtin_inff();  // render.cu:585-586
-    int last_j = -1;
+    int last_j = -1;  // list positions count from the tile's start
     bool active = p.valid;
     while (true) {
         const bool want = active && s.alpha > a.thr && s.blended < a.max_layers;  // render.cu:588
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                 real b0, b1, b2;
                 bary_apply(r.m, p.px, p.py, b0, b1, b2);
                 const real pd = interp_w(b0, b1, b2, r.z[0], r.z[1], r.z[2], r.w[0], r.w[1], r.w[2]);  // render.cu:404
-                const int j = batch + e;
+                const int j = batch + e - start;
                 if (pd < last_depth) continue;
                 if (pd == last_depth && j <= last_j) continue;
                 topk_insert(tk, cap, found, pd, j);
@@ -247,7 +252,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                     BlendRecord r[kGatherAhead];
 #pragma unroll
                     for (int u = 0; u < kGatherAhead; u++) {
-                        const int rel = tk.j(min(i0 + u, todo - 1)) - start;
+                        const int rel = tk.j(min(i0 + u, todo - 1));
                         if (rel < n_rows) {
                             real *w = reinterpret_cast<real *>(&r[u]);
 #pragma unroll
@@ -262,7 +267,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
                         real b0, b1, b2;
                         bary_apply(r[u].m, p.px, p.py, b0, b1, b2);
                         if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
-                        if (out.fragments) out.fragments[(int64_t)s.blended * ((int64_t)a.W * a.H) + p.index] = tk.j(i0 + u) - start;
+                        if (out.fragments) out.fragments[(int64_t)s.blended * ((int64_t)a.W * a.H) + p.index] = tk.j(i0 + u);
                         blend_fragment(s, r[u], b0, b1, b2);
                     }
                 }
@@ -274,7 +279,51 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
             }
         }
     }
-    if (p.valid) write_pixel(out, p, s, last_j >= 0 ? last_j - start + 1 : 0, last_depth);
+    if (p.valid) write_pixel(out, p, s, last_j + 1, last_depth);
+}
+
+// One workgroup per tile.  With 16-bit positions the tiles whose lists are too long for them are left to
+// forward_pixel_order_long_lists_kernel.
+template <int kStage, typename Pos>
+__global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(RasterArgs a, ForwardOut out) {
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    __shared__ uint8_t s_touch[kStage];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    if (sizeof(Pos) < sizeof(int) && a.offsets[tile + 1] - a.offsets[tile] > kShortList) return;
+    pixel_order_tile<kStage, Pos>(a, out, blockIdx.x, blockIdx.y, gridDim.x, s_dyn, s_touch, s_rects);
+}
+
+// The tiles whose lists are longer than kShortList, with int positions: few or none, so a small grid
+// looks through the tiles' list lengths (a workgroup through its share of the tiles, one tile per thread at a
+// time) and takes those.
+__global__ __launch_bounds__(kTileThreads) void forward_pixel_order_long_lists_kernel(RasterArgs a, ForwardOut out, int tiles_x,
+                                                                                      int tiles_y) {
+    extern __shared__ __align__(16) unsigned char s_dyn[];
+    __shared__ uint8_t s_touch[kSelectBatch];
+    __shared__ WaveRect s_rects[kMaxTileWaves];
+    __shared__ uint64_t s_votes[kMaxTileWaves];
+    const int tiles = tiles_x * tiles_y;
+    const int share = (tiles + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int first = blockIdx.x * share, past = min(first + share, tiles);
+    const int n_waves = blockDim.x / kWave;
+    for (int base = first; base < past; base += blockDim.x) {
+        const int mine = base + (int)threadIdx.x;
+        const bool is_long = mine < past && a.offsets[mine + 1] - a.offsets[mine] > kShortList;
+        const uint64_t vote = __builtin_amdgcn_ballot_w64(is_long);
+        __syncthreads();  // the round before is done with the votes
+        if ((threadIdx.x & (kWave - 1)) == 0) s_votes[threadIdx.x / kWave] = vote;
+        __syncthreads();
+        for (int w = 0; w < n_waves; w++) {
+            uint64_t todo = s_votes[w];
+            while (todo) {  // the same for the whole workgroup
+                const int tile = base + w * kWave + __builtin_ctzll(todo);
+                todo &= todo - 1;
+                __syncthreads();  // the tile before is done with the LDS
+                pixel_order_tile<kSelectBatch, int>(a, out, tile % tiles_x, tile / tiles_x, tiles_x, s_dyn, s_touch, s_rects);
+            }
+        }
+    }
 }
 
 TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads) {
@@ -307,8 +356,8 @@ int pixel_order_threads(int preferred) {
     return override ? override : preferred;
 }
 
-size_t pixel_order_lds_bytes(int n_threads, int staged_entries) {
-    return sizeof(DepthRecord) * staged_entries + (size_t)kLayers * n_threads * (sizeof(real) + sizeof(int));
+size_t pixel_order_lds_bytes(int n_threads, int staged_entries, size_t position_bytes) {
+    return sizeof(DepthRecord) * staged_entries + (size_t)kLayers * n_threads * (sizeof(real) + position_bytes);
 }
 
 // Dynamic LDS beyond 64 KB has to be enabled per kernel once.
@@ -386,8 +435,21 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         return check_launch("forward_tile_order_kernel");
     }
     const size_t lds = pixel_order_lds_bytes(n_threads, kSelectBatch);
-    static size_t lds_reserved = 0;
-    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatch>, lds, &lds_reserved)) return e;
-    TG_LAUNCH_AS("forward_pixel_order_kernel", forward_pixel_order_kernel<kSelectBatch>, grid, dim3(n_threads), lds, s, a, o);
-    return check_launch("forward_pixel_order_kernel");
+    // Depth bounds make the batches jump in steps of kSelectBatch, so they go with the int positions.
+    const bool split = !a.batch_bounds && n_threads >= kSelectBatchShort;
+    static size_t lds_reserved = 0, lds_reserved_long = 0;
+    if (!split) {
+        if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatch, int>, lds, &lds_reserved)) return e;
+        TG_LAUNCH_AS("forward_pixel_order_kernel", (forward_pixel_order_kernel<kSelectBatch, int>), grid, dim3(n_threads), lds, s, a, o);
+        return check_launch("forward_pixel_order_kernel");
+    }
+    const size_t lds_short = pixel_order_lds_bytes(n_threads, kSelectBatchShort, sizeof(uint16_t));
+    TG_LAUNCH_AS("forward_pixel_order_kernel", (forward_pixel_order_kernel<kSelectBatchShort, uint16_t>), grid, dim3(n_threads),
+                 lds_short, s, a, o);
+    if (int e = check_launch("forward_pixel_order_kernel")) return e;
+    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_long_lists_kernel, lds, &lds_reserved_long)) return e;
+    const int tiles = (int)(grid.x * grid.y);
+    TG_LAUNCH(forward_pixel_order_long_lists_kernel, dim3(min(tiles, kLongListGroups), 1, grid.z), dim3(n_threads), lds, s, a, o,
+              (int)grid.x, (int)grid.y);
+    return check_launch("forward_pixel_order_long_lists_kernel");
 }

@@ -41,7 +41,7 @@ struct PixelCoord {
     real px, py;
 };
 
-__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
+__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a, int tile_x, int tile_y) {
     PixelCoord p;
     const int t = blockIdx.z * blockDim.x + threadIdx.x;
     int lx, ly;
@@ -55,14 +55,15 @@ __device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) {
         lx = t % a.tw;
         ly = t / a.tw;
     }
-    p.ix = blockIdx.x * a.tw + lx;
-    p.iy = blockIdx.y * a.th + ly;
+    p.ix = tile_x * a.tw + lx;
+    p.iy = tile_y * a.th + ly;
     p.valid = (t < a.tw * a.th) && p.ix < a.W && p.iy < a.H;  // render.cu:554
     p.index = p.iy * a.W + p.ix;
     p.px = pixel_ndc(p.ix, a.W);
     p.py = pixel_ndc(p.iy, a.H);
     return p;
 }
+__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) { return pixel_of_thread(a, blockIdx.x, blockIdx.y); }
 
 // Everything process_forward (render.cu:417-453) reads for one list entry.
 struct alignas(16) BlendRecord {
@@ -177,7 +178,7 @@ __device__ __forceinline__ void blend_fragment(PixelState &s, const BlendRecord 
 struct TileLaunch { dim3 grid; int threads; };
 TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_threads);
 int pixel_order_threads(int preferred);
-size_t pixel_order_lds_bytes(int n_threads, int staged_entries);
+size_t pixel_order_lds_bytes(int n_threads, int staged_entries, size_t position_bytes = sizeof(int));
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
 int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
 
@@ -290,12 +291,14 @@ __device__ __forceinline__ int pop_lowest(uint64_t m[kWords]) {
 
 // Per-pixel candidate lists of the per-pixel-sort mode live in LDS, slot-major:
 // entry `slot` of thread `t` is at [slot * n_threads + t] (conflict-free).
-struct TopK {
+template <typename Pos>
+struct TopKOf {
     real *depth;
-    int *pos;
+    Pos *pos;
     int n_threads;
     __device__ __forceinline__ real &d(int slot) const { return depth[slot * n_threads + threadIdx.x]; }
-    __device__ __forceinline__ int &j(int slot) const { return pos[slot * n_threads + threadIdx.x]; }
+    __device__ __forceinline__ Pos &j(int slot) const { return pos[slot * n_threads + threadIdx.x]; }
 };
+using TopK = TopKOf<int>;
 
 }  // namespace tg
