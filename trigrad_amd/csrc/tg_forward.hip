@@ -444,6 +444,10 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         return check_launch("forward_pixel_order_kernel");
     }
     const size_t lds_short = pixel_order_lds_bytes(n_threads, kSelectBatchShort, sizeof(uint16_t));
+    static size_t lds_reserved_short = 0;
+    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatchShort, uint16_t>, lds_short,
+                            &lds_reserved_short))
+        return e;
     TG_LAUNCH_AS("forward_pixel_order_kernel", (forward_pixel_order_kernel<kSelectBatchShort, uint16_t>), grid, dim3(n_threads),
                  lds_short, s, a, o);
     if (int e = check_launch("forward_pixel_order_kernel")) return e;
