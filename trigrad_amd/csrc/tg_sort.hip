@@ -715,23 +715,39 @@ __device__ void segment_sort_through_memory(uint64_t *keys, uint32_t *vals, uint
     }
 }
 
-// Segments longer than kSegMediumCap: the workgroups take them in turn.
+// Segments longer than kSegMediumCap: few or none, so a workgroup looks through the lengths of its share of the
+// segments, one segment per thread at a time, and takes the long ones in turn.
 __global__ __launch_bounds__(kSortThreads, 2) void segment_sort_large_kernel(uint64_t *keys, uint32_t *vals, uint64_t *keys_alt,
                                                                              uint32_t *vals_alt, const int32_t *__restrict__ offsets,
                                                                              int n_segments) {
     __shared__ SegLds lds;
     __shared__ uint32_t ex_keys[kSegLargeCap], ex_vals[kSegLargeCap];
-    for (int seg = blockIdx.x; seg < n_segments; seg += gridDim.x) {
-        const int64_t start = offsets[seg];
-        const int n = offsets[seg + 1] - offsets[seg];
-        if (n <= kSegMediumCap) continue;
-        if (n <= kSortThreads * 16)
-            segment_sort_in_lds<16>(keys, vals, start, n, lds, ex_keys, ex_vals);
-        else if (n <= kSegLargeCap)
-            segment_sort_in_lds<kSegLargeItems>(keys, vals, start, n, lds, ex_keys, ex_vals);
-        else
-            segment_sort_through_memory(keys, vals, keys_alt, vals_alt, start, n, lds, ex_keys, ex_keys + kRadix);
-        __syncthreads();  // the next segment reuses the LDS
+    __shared__ uint64_t s_votes[kSortWaves];
+    // workgroup b looks at the segments b, b + gridDim.x, ...: long segments that are neighbours go to different workgroups
+    const int grid = (int)gridDim.x;
+    for (int base = 0; (int64_t)base * grid < n_segments; base += kSortThreads) {
+        const int mine = (base + (int)threadIdx.x) * grid + (int)blockIdx.x;
+        const bool is_long = mine < n_segments && offsets[mine + 1] - offsets[mine] > kSegMediumCap;
+        const uint64_t vote = __builtin_amdgcn_ballot_w64(is_long);
+        __syncthreads();  // the round before is done with the votes, the segment before with the LDS
+        if ((threadIdx.x & (kWave - 1)) == 0) s_votes[threadIdx.x / kWave] = vote;
+        __syncthreads();
+        for (int w = 0; w < kSortWaves; w++) {
+            uint64_t todo = s_votes[w];
+            while (todo) {  // the same for the whole workgroup
+                const int seg = (base + w * kWave + __builtin_ctzll(todo)) * grid + (int)blockIdx.x;
+                todo &= todo - 1;
+                const int64_t start = offsets[seg];
+                const int n = offsets[seg + 1] - offsets[seg];
+                if (n <= kSortThreads * 16)
+                    segment_sort_in_lds<16>(keys, vals, start, n, lds, ex_keys, ex_vals);
+                else if (n <= kSegLargeCap)
+                    segment_sort_in_lds<kSegLargeItems>(keys, vals, start, n, lds, ex_keys, ex_vals);
+                else
+                    segment_sort_through_memory(keys, vals, keys_alt, vals_alt, start, n, lds, ex_keys, ex_keys + kRadix);
+                __syncthreads();  // the next segment reuses the LDS
+            }
+        }
     }
 }
 
