@@ -226,25 +226,61 @@ def bin_setup(vertices, indices, width, height, tile_width, tile_height, with_he
                 geometry=(width, height, tile_width, tile_height), bits=bits)
 
 
-def build_tile_lists(setup, n_keys, emit_only=False):
+_key_count_hint = {}  # device index -> K of the device's last frame
+
+
+def prepare_tile_lists(setup):
+    """Buffers for build_tile_lists, allocated before K is known: for as many keys as the device's last frame had
+    plus an eighth.  The host has nothing to do while it waits for K, and every allocation made after K has
+    arrived is time the device idles.  None without a last frame (or for the double build)."""
+    hint = _key_count_hint.get(setup["records"].device.index)
+    if hint is None or setup["bits"] != 32:
+        return None
+    capacity = hint + hint // 8 + 1024
+    return _tile_list_buffers(setup, capacity)
+
+
+def _tile_list_buffers(setup, capacity):
+    lib = _lib.load(setup["bits"])
+    dev = setup["records"].device
+    T = num_tiles(*setup["geometry"])
+    ws_bytes = int(lib.tg_build_tile_lists_workspace_bytes(capacity, T))
+    return dict(capacity=capacity, ws_bytes=ws_bytes,
+                keys=torch.empty((capacity,), dtype=torch.int64, device=dev),
+                values=torch.empty((capacity,), dtype=torch.int32, device=dev),
+                keys_alt=torch.empty((capacity,), dtype=torch.int64, device=dev),
+                values_alt=torch.empty((capacity,), dtype=torch.int32, device=dev),
+                offsets=torch.empty((T + 1,), dtype=torch.int32, device=dev),
+                status=torch.empty((1,), dtype=torch.int32, device=dev),
+                ws=torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev))
+
+
+def build_tile_lists(setup, n_keys, emit_only=False, prepared=None):
     """bin_setup's result + K -> (sorted_keys, sorted_ids, status (1,) int32, offsets (T+1,) int32);
-    emit_only: (keys, ids, status, None) in emission order (float64: 2K keys, depth keys then tile ids)."""
+    emit_only: (keys, ids, status, None) in emission order (float64: 2K keys, depth keys then tile ids).
+    prepared: prepare_tile_lists' buffers, used if they hold n_keys keys."""
     bits = setup["bits"]
     lib = _lib.load(bits)
     records, tri_offsets, heads, frame = setup["records"], setup["tri_offsets"], setup["heads"], setup["frame"]
     width, height, tile_width, tile_height = setup["geometry"]
     dev = records.device
-    T = num_tiles(width, height, tile_width, tile_height)
-    keys = torch.empty((n_keys * (2 if bits == 64 else 1),), dtype=torch.int64, device=dev)
-    values = torch.empty((n_keys,), dtype=torch.int32, device=dev)
-    status = torch.empty((1,), dtype=torch.int32, device=dev)
-    keys_alt = values_alt = offsets = ws = None
-    ws_bytes = 0
-    if not emit_only:
-        keys_alt, values_alt = torch.empty_like(keys), torch.empty_like(values)
-        offsets = torch.empty((T + 1,), dtype=torch.int32, device=dev)
-        ws_bytes = int(lib.tg_build_tile_lists_workspace_bytes(n_keys, T))
-        ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    _key_count_hint[dev.index] = n_keys
+    if emit_only or bits != 32:
+        keys = torch.empty((n_keys * (2 if bits == 64 else 1),), dtype=torch.int64, device=dev)
+        values = torch.empty((n_keys,), dtype=torch.int32, device=dev)
+        status = torch.empty((1,), dtype=torch.int32, device=dev)
+        keys_alt = values_alt = offsets = ws = None
+        ws_bytes = 0
+        if not emit_only:
+            T = num_tiles(width, height, tile_width, tile_height)
+            keys_alt, values_alt = torch.empty_like(keys), torch.empty_like(values)
+            offsets = torch.empty((T + 1,), dtype=torch.int32, device=dev)
+            ws_bytes = int(lib.tg_build_tile_lists_workspace_bytes(n_keys, T))
+            ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    else:
+        b = prepared if prepared is not None and n_keys <= prepared["capacity"] else _tile_list_buffers(setup, n_keys)
+        keys, values, keys_alt, values_alt = b["keys"], b["values"], b["keys_alt"], b["values_alt"]
+        offsets, status, ws, ws_bytes = b["offsets"], b["status"], b["ws"], b["ws_bytes"]
     in_alt = C.c_int(0)
     with _on_device(dev):
         _lib.check(lib.tg_build_tile_lists(_ptr(records), _ptr(tri_offsets), tri_offsets.numel(), n_keys,
@@ -253,7 +289,9 @@ def build_tile_lists(setup, n_keys, emit_only=False):
                                            _ptr(offsets), _ptr(ws), ws_bytes, _ptr(status), int(bool(emit_only)), C.byref(in_alt),
                                            _stream(records)), "tg_build_tile_lists", bits)
     if in_alt.value:
-        return keys_alt, values_alt, status, offsets
+        keys, values = keys_alt, values_alt
+    if keys.numel() != n_keys * (2 if bits == 64 else 1):
+        keys, values = keys[:n_keys], values[:n_keys]  # buffers made for more keys
     return keys, values, status, offsets
 
 
@@ -419,7 +457,7 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
         setup = bin_setup(vertices, indices, width, height, tile_width, tile_height)
-        bary_transforms = None
+        bary_transforms = prepared = None
         if disable_timing:
             # K travels to pinned host memory while the device already computes the bary matrices, which do
             # not depend on it; the host waits for the copy only (with stage timings the reference's order is kept)
@@ -428,6 +466,7 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
             arrived = torch.cuda.Event()
             arrived.record()
             bary_transforms = cartesian_to_bary(vertices, indices)
+            prepared = prepare_tile_lists(setup)
             arrived.synchronize()
         else:
             host = setup["total_and_status"].cpu()
@@ -435,7 +474,7 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
         if st != 0:
             raise RuntimeError("tg_bin_setup: look-back wait timed out")
         if bits == 32 and disable_timing:
-            keys, sorted_ids, sort_status, offsets = build_tile_lists(setup, K)
+            keys, sorted_ids, sort_status, offsets = build_tile_lists(setup, K, prepared=prepared)
         else:
             # the stages apart, so that their times are the reference's (render.cu:733-745); the double build's
             # depth keys take 64 bits and are sorted in two rounds
