@@ -104,23 +104,24 @@ def _long_list_scene():
     return scene
 
 
-@pytest.mark.parametrize("mode", ["A_default", "A_40_layers", "B_3_layers"])
-def test_tile_list_longer_than_16_bit_positions(mode, cuda, oracle):
+@pytest.mark.parametrize("mode,tile", [("A_default", 16), ("A_40_layers", 16), ("B_3_layers", 16), ("A_default", 32)])
+def test_tile_list_longer_than_16_bit_positions(mode, tile, cuda, oracle):
     import torch
     from trigrad_amd import _C
     scene = _long_list_scene()
     m = MODES[mode]
-    d, want, got, ml = _forward_both(scene, 16, 16, m, cuda, oracle)
+    d, want, got, ml = _forward_both(scene, tile, tile, m, cuda, oracle)
     lengths = np.diff(want["offsets"])
-    assert lengths.max() > 65535 and lengths.min() < 65535
+    # 16x16: one long list next to short ones; 32x32: the one tile is four workgroups on the long list
+    assert lengths.max() > 65535 and (tile == 32 or lengths.min() < 65535)
     _check_forward(f"long list/{mode}", want, got)
     gi, gd = _grad_inputs(scene, 9, True)
     gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
-                                        32, 32, 16, 16, m["per_pixel_sort"], ml, literal=False)
+                                        32, 32, tile, tile, m["per_pixel_sort"], ml, literal=False)
     image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
     out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                              d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, 32, 32,
-                             16, 16, 1 / 256, m["per_pixel_sort"], ml, resume=resume)
+                             tile, tile, 1 / 256, m["per_pixel_sort"], ml, resume=resume)
     for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
         scale = float(np.abs(w).max())
         assert_close(f"long list/{mode}: {label}", g.cpu().numpy().astype(np.float64), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * scale)
