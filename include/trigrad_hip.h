@@ -285,6 +285,13 @@ int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, 
                        tg_real *grad_colors, tg_real *grad_opacities, int vertex_stride, int color_stride,
                        int opacity_stride, void *stream);
 
+/* The (V,8) block that tg_render_backward accumulates into with strides
+ * (8, 8, 8) -> the three dense arrays the reference's render_backward returns
+ * (render.cu:765-804: grad_vertices (V,4), grad_colors (V,3), grad_opacities
+ * (V)): scalars 0..3 of a vertex's row, 4..6 and 7.  One pass over the block. */
+int tg_split_gradient_block(const tg_real *block, int64_t n_vertices, tg_real *grad_vertices, tg_real *grad_colors,
+                            tg_real *grad_opacities, void *stream);
+
 /* ---- host-side component hooks ---------------------------------------------- */
 
 /* HOST pointers, run on the CPU.  The reference exports the same six functions

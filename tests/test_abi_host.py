@@ -55,6 +55,9 @@ def test_host_side_helpers_and_argument_rejection(bits):
     assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 11)) == -1
     assert b"max_layers" in lib.tg_last_error()
     assert lib.tg_render_backward(*([None] * 17), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, 4, 3, 1, None) == -1
+    assert lib.tg_split_gradient_block(None, 5, None, None, None, None) == -1 and b"null pointer" in lib.tg_last_error()
+    assert lib.tg_split_gradient_block(None, -1, None, None, None, None) == -1
+    assert lib.tg_split_gradient_block(None, 0, None, None, None, None) == 0
     assert lib.tg_hit_mask_words(6400, 64, 64, 16, 16) == 16 + (100 + 16 + 1) * 256  # a word per workgroup, then the chunks
     assert lib.tg_list_bound_words(6400, 16) == 25 + 16 + 1
     assert lib.tg_list_bounds(None, 0, None, 0, None, None, None, 0, None, None, None, None) == -1

@@ -609,7 +609,13 @@ def render_backward(grad_output, grad_depthmap, vertices, indices, colors, opaci
             *[_ptr(t) for t in tensors], _ptr(last_depth), _ptr(fragments), _ptr(hit_masks), width, height, tile_width, tile_height,
             float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers), _ptr(grad_vertices), _ptr(grad_colors),
             _ptr(grad_opacities), *strides, _stream(vertices)), "tg_render_backward", bits)
-        if strides != (4, 3, 1):
+        if strides == (8, 8, 8):
+            grad_vertices = torch.empty((V, 4), dtype=vertices.dtype, device=dev)
+            grad_colors = torch.empty((V, 3), dtype=vertices.dtype, device=dev)
+            grad_opacities = torch.empty((V,), dtype=vertices.dtype, device=dev)
+            _lib.check(lib.tg_split_gradient_block(_ptr(b8), V, _ptr(grad_vertices), _ptr(grad_colors), _ptr(grad_opacities),
+                                                   _stream(vertices)), "tg_split_gradient_block", bits)
+        elif strides != (4, 3, 1):
             grad_vertices, grad_colors, grad_opacities = (grad_vertices.contiguous(), grad_colors.contiguous(),
                                                           grad_opacities.contiguous())
     return grad_vertices, grad_colors, grad_opacities

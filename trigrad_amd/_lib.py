@@ -53,6 +53,7 @@ SIGNATURES = {
     "tg_hit_mask_words": (_sz, [_i64, _i, _i, _i, _i]),
     "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "tg_render_backward": (_i, [_p] * 17 + [_i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _i, _i, _i, _p]),
+    "tg_split_gradient_block": (_i, [_p, _i64, _p, _p, _p, _p]),
     "tg_barycentric": (None, [_p] * 5),
     "tg_barycentric_backward": (None, [_p] * 6),
     "tg_interpolate3_scalar": (_f, [_p, _f, _f, _f, _p]),

@@ -943,6 +943,21 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     }
 }
 
+// The three gradient arrays out of the (V,8) block the per-pixel-order kernels accumulate into:
+// one read of the block instead of the three strided ones that three separate copies make.
+__global__ __launch_bounds__(256) void split_gradient_block_kernel(const real4 *__restrict__ block, int64_t n_vertices,
+                                                                   real4 *__restrict__ grad_vertices, real *__restrict__ grad_colors,
+                                                                   real *__restrict__ grad_opacities) {
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v >= n_vertices) return;
+    const real4 position = block[2 * v], rest = block[2 * v + 1];
+    grad_vertices[v] = position;
+    grad_colors[3 * v] = rest.x;
+    grad_colors[3 * v + 1] = rest.y;
+    grad_colors[3 * v + 2] = rest.z;
+    grad_opacities[v] = rest.w;
+}
+
 size_t backward_pixel_order_lds_bytes(int n_threads) { return pixel_order_lds_bytes(n_threads, kBatch) + (size_t)kAccWindow * kTerms * sizeof(real); }
 
 }  // namespace tg
@@ -1014,4 +1029,24 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
     TG_LAUNCH_BACKWARD(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds);
     return check_launch("backward_pixel_order_kernel");
 #undef TG_LAUNCH_BACKWARD
+}
+
+extern "C" int tg_split_gradient_block(const real *block, int64_t n_vertices, real *grad_vertices, real *grad_colors,
+                                       real *grad_opacities, void *stream) {
+    if (n_vertices < 0 || n_vertices > (int64_t)0x7fffffff * 256) {
+        set_error("tg_split_gradient_block: n_vertices out of range");
+        return TG_E_ARG;
+    }
+    if (n_vertices == 0) return 0;
+    if (!block || !grad_vertices || !grad_colors || !grad_opacities) {
+        set_error("tg_split_gradient_block: null pointer");
+        return TG_E_ARG;
+    }
+    if (((uintptr_t)block & 15) || ((uintptr_t)grad_vertices & 15)) {
+        set_error("tg_split_gradient_block: block and grad_vertices must be 16-byte aligned");
+        return TG_E_ARG;
+    }
+    TG_LAUNCH(split_gradient_block_kernel, dim3((unsigned)ceil_div64(n_vertices, 256)), dim3(256), 0, (hipStream_t)stream,
+              (const real4 *)block, n_vertices, (real4 *)grad_vertices, grad_colors, grad_opacities);
+    return check_launch("split_gradient_block_kernel");
 }
