@@ -474,9 +474,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const int n_waves = blockDim.x / kWave;
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const TileId tile_id = tile_of_workgroup<kTileBandBackward>();
+    const int tile = tile_id.index;
     const int start = a.offsets[tile];
-    const PixelCoord p = pixel_of_thread(a);
+    const PixelCoord p = pixel_of_thread(a, tile_id);
     const TermLane tl = term_lane<kLayout>(g, lane);
     uint64_t *ballots = s_ballot[wave];
     uint32_t *bases = s_base[wave];
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
     if (p.valid) st = load_back_state(g, p);
     int tile_last;
     if (saved_masks) {
-        tile_last = (int)g.hit_masks[hit_mask_head_index()];
+        tile_last = (int)g.hit_masks[hit_mask_head_index(tile)];
     } else {
         if (tid == 0) s_last = 0;
         publish_wave_rect(p, s_rects);  // only the repeated inside tests cull by wave rectangle
@@ -693,9 +694,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
     const int n_waves = blockDim.x / kWave;
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const TileId tile_id = tile_of_workgroup<kTileBandBackward>();
+    const int tile = tile_id.index;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
-    const PixelCoord p = pixel_of_thread(a);
+    const PixelCoord p = pixel_of_thread(a, tile_id);
     publish_wave_rect(p, s_rects);
     const int n_acc = min(end - start, kAccWindow);
     for (int i = tid; i < n_acc * kTerms; i += blockDim.x) s_acc[i] = 0.0f;
@@ -814,9 +816,10 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const TileId tile_id = tile_of_workgroup<kTileBandBackward>();
+    const int tile = tile_id.index;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
-    const PixelCoord p = pixel_of_thread(a);
+    const PixelCoord p = pixel_of_thread(a, tile_id);
     const int rel_bits = 32 - __builtin_clz(max(end - start - 1, 1));  // bits that tell two list positions apart
     real *terms = s_term[wave];
     int *rels = s_rel[wave];

@@ -51,9 +51,10 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
     const int n_waves = blockDim.x / kWave;
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const TileId tile_id = tile_of_workgroup<kTileBandForward>();
+    const int tile = tile_id.index;
     const int start = a.offsets[tile], end = a.offsets[tile + 1];
-    const PixelCoord p = pixel_of_thread(a);
+    const PixelCoord p = pixel_of_thread(a, tile_id);
     publish_wave_rect(p, s_rects);
     uint64_t *const masks = out.hit_masks ? out.hit_masks + hit_mask_head_words() : nullptr;
 
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
         for (int off = 32; off > 0; off >>= 1) wave_last = max(wave_last, __shfl_xor(wave_last, off, kWave));
         if ((tid & (kWave - 1)) == 0 && wave_last > 0) atomicMax(&s_last, wave_last);
         __syncthreads();
-        if (tid == 0) out.hit_masks[hit_mask_head_index()] = (uint64_t)s_last;
+        if (tid == 0) out.hit_masks[hit_mask_head_index(tile)] = (uint64_t)s_last;
     }
 }
 
@@ -289,9 +290,9 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
     extern __shared__ __align__(16) unsigned char s_dyn[];
     __shared__ uint8_t s_touch[kStage];
     __shared__ WaveRect s_rects[kMaxTileWaves];
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    if (sizeof(Pos) < sizeof(int) && a.offsets[tile + 1] - a.offsets[tile] > kShortList) return;
-    pixel_order_tile<kStage, Pos>(a, out, blockIdx.x, blockIdx.y, gridDim.x, s_dyn, s_touch, s_rects);
+    const TileId tile = tile_of_workgroup<kTileBandForward>();
+    if (sizeof(Pos) < sizeof(int) && a.offsets[tile.index + 1] - a.offsets[tile.index] > kShortList) return;
+    pixel_order_tile<kStage, Pos>(a, out, tile.x, tile.y, gridDim.x, s_dyn, s_touch, s_rects);
 }
 
 // The tiles whose lists are longer than kShortList, with int positions: few or none, so a small grid

@@ -63,7 +63,46 @@ __device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a, int t
     p.py = pixel_ndc(p.iy, a.H);
     return p;
 }
-__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a) { return pixel_of_thread(a, blockIdx.x, blockIdx.y); }
+
+// The tile a workgroup of a (tiles_x, tiles_y, parts) launch takes.  Workgroups go to the eight XCDs of the device in
+// turn in the order of their linear index, and every XCD has an L2 of its own; neighbouring tiles share list
+// entries (a triangle that covers two tiles is in both lists), vertices and matrices.  So the workgroups
+// that reach one XCD take consecutive tiles of an order that keeps neighbours together: bands of kTileBand
+// tile rows, column by column inside a band.  XCD k gets the k-th eighth of that order, and the workgroups that
+// run there at one time cover a compact block of the image.
+#ifndef TG_XCD_TILES
+#define TG_XCD_TILES 1
+#endif
+#ifndef TG_TILE_BAND_FORWARD
+#define TG_TILE_BAND_FORWARD 8
+#endif
+#ifndef TG_TILE_BAND_BACKWARD
+#define TG_TILE_BAND_BACKWARD 1
+#endif
+constexpr int kXcds = 8;
+constexpr int kTileBandForward = TG_TILE_BAND_FORWARD, kTileBandBackward = TG_TILE_BAND_BACKWARD;
+struct TileId { int x, y, index; };
+template <int kTileBand>
+__device__ __forceinline__ TileId tile_of_workgroup() {
+    const int tiles_x = (int)gridDim.x, tiles_y = (int)gridDim.y, n = tiles_x * tiles_y;
+    const int linear = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+    TileId t;
+#if TG_XCD_TILES
+    const int per = n / kXcds, rest = n % kXcds;
+    const int xcd = linear % kXcds, turn = linear / kXcds;
+    const int place = xcd < rest ? xcd * (per + 1) + turn : rest * (per + 1) + (xcd - rest) * per + turn;
+    const int band = place / (kTileBand * tiles_x), within = place - band * (kTileBand * tiles_x);
+    const int rows = min(kTileBand, tiles_y - band * kTileBand);
+    t.x = within / rows;
+    t.y = band * kTileBand + within % rows;
+#else
+    t.x = linear % tiles_x;
+    t.y = linear / tiles_x;
+#endif
+    t.index = t.y * tiles_x + t.x;
+    return t;
+}
+__device__ __forceinline__ PixelCoord pixel_of_thread(const RasterArgs &a, const TileId &t) { return pixel_of_thread(a, t.x, t.y); }
 
 // Everything process_forward (render.cu:417-453) reads for one list entry.
 struct alignas(16) BlendRecord {
@@ -134,9 +173,7 @@ __device__ __forceinline__ void gather_depth(const RasterArgs &a, int j, DepthRe
 __device__ __forceinline__ int64_t hit_mask_chunk(int start, int tile, int relative_position) {
     return (int64_t)(start >> 6) + tile + (relative_position >> 6);
 }
-__device__ __forceinline__ int64_t hit_mask_head_index() {
-    return ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * gridDim.z + blockIdx.z;
-}
+__device__ __forceinline__ int64_t hit_mask_head_index(int tile) { return (int64_t)tile * gridDim.z + blockIdx.z; }
 __device__ __forceinline__ int64_t hit_mask_head_words() { return (int64_t)gridDim.x * gridDim.y * gridDim.z; }
 
 // Batch bounds: word batch_bound_index(start, tile, p) holds, for the tile whose
