@@ -237,6 +237,8 @@ def prepare_tile_lists(setup):
     if hint is None or setup["bits"] != 32:
         return None
     capacity = hint + hint // 8 + 1024
+    if int(_lib.load(32).tg_build_tile_lists_workspace_bytes(capacity, num_tiles(*setup["geometry"]))) == 0:
+        return None  # more keys than the sort takes: leave it to the call that knows K
     return _tile_list_buffers(setup, capacity)
 
 
