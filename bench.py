@@ -127,7 +127,7 @@ def main():
     sort_kernels = ["fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel",
                     "segment_sort_small_kernel", "segment_sort_large_kernel"]
     bin_sort_kernels = ["bin_count_kernel", "scan_init_kernel", "scan_lookback_kernel", "bin_emit_kernel", "bin_init_kernel",
-                        "bin_setup_kernel", "bin_emit_records_kernel", "tile_ranges_kernel"] + sort_kernels
+                        "bin_setup_kernel", "bin_emit_records_kernel", "frame_scan_kernel", "frame_emit_kernel", "tile_ranges_kernel"] + sort_kernels
     bin_sort_ms = sum(per_step.get(k, 0.0) for k in bin_sort_kernels)
     bin_sort_bytes = 136.0 * M + 28.0 * K + 24.0 * passes * K + 4.0 * (T + 1)
     sort_ms = sum(per_step.get(k, 0.0) for k in sort_kernels)

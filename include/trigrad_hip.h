@@ -204,6 +204,52 @@ int tg_build_tile_lists(const tg_real *records, const uint32_t *tri_offsets, int
                         int32_t *offsets, void *workspace, size_t workspace_bytes, uint32_t *status, int emit_only,
                         int *result_in_alt, void *stream);
 
+/* ---- (1)-(3) as the frame runs them now: no wait for the host inside the binning ---- */
+
+/* tg_bin_frame = tg_bin_count + tg_scan_exclusive_u32 + tg_bin_emit in one call
+ * and two launches (count_per_tile, the cumsum of per_tile_lists and
+ * fill_per_tile_lists_kernel, render.cu:90-139, 202-270, 290-308): keys and
+ * values as tg_bin_emit leaves them, total_and_status[0] = K.  The emission
+ * reads K on the device, so the host does not have to know it in between: the
+ * key buffers are the caller's guess, a key whose position is key_capacity or
+ * more is not written, K is exact either way, and a caller who finds
+ * K > key_capacity calls again with larger buffers.  Float build only, up to
+ * 2^21 tiles (tg_bin_frame_supported; tg_bin_setup + tg_build_tile_lists take
+ * the rest).
+ *
+ * frame: tg_bin_frame_workspace_bytes() bytes, 256-byte aligned, ZERO before the
+ * first call that uses it; every call leaves it ready for the next.  It holds
+ * what the two launches hand each other (per-triangle records as tg_bin_setup
+ * makes them) and what calls share.  epoch: its low 30 bits must not be 0,
+ * must differ from those of every earlier call on this frame state since it
+ * was zeroed, and its lowest bit must differ from the previous call's (count
+ * up by one).  The scan marks what it publishes with the epoch, so nothing is
+ * cleared between calls.  One call at a time per frame state.  A wait for
+ * another workgroup that expires (see TG_STATUS_*) writes `epoch` to
+ * total_and_status[1], which is not written otherwise: pass a word that holds
+ * something else.
+ *
+ * On the side the first launch zeroes zero_bytes bytes at `zero` (pass the
+ * workspace of the tg_build_frame_lists call that follows, sized for
+ * key_capacity keys) and *clear_word (its status word); both may be NULL / 0.
+ *
+ * tg_build_frame_lists = tg_sort_tile_lists on the keys tg_bin_frame emitted
+ * (sort_depth_ranges and the offsets of per_tile_lists, render.cu:272-308),
+ * same results bit for bit.  It takes the digit totals of the tile passes from
+ * the frame state (tg_bin_frame counted them for `epoch`), so it reads the keys
+ * for no histogram.  workspace: tg_build_frame_lists_workspace_bytes(), zeroed
+ * by the tg_bin_frame call; status: cleared by that call. */
+int tg_bin_frame_supported(int width, int height, int tile_w, int tile_h);
+size_t tg_bin_frame_workspace_bytes(int32_t n_triangles, int64_t key_capacity, int width, int height, int tile_w, int tile_h);
+int tg_bin_frame(const tg_real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width,
+                 int height, int tile_w, int tile_h, uint64_t *keys, uint32_t *values, int64_t key_capacity,
+                 uint32_t *total_and_status, void *frame, size_t frame_bytes, uint32_t epoch, void *zero,
+                 size_t zero_bytes, uint32_t *clear_word, void *stream);
+size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int n_tiles);
+int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int n_tiles, uint64_t *keys, uint32_t *values,
+                         uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
+                         size_t workspace_bytes, uint32_t *status, int *result_in_alt, void *stream);
+
 /* ---- bary matrices ---------------------------------------------------------- */
 
 /* Row-major 3x3 cartesian-to-barycentric matrix per triangle, out is (M,3,3).

@@ -9,6 +9,7 @@ current torch stream.  torch is used for device memory and streams only.
 and the individual stages are exposed as functions for tests and benchmarks.
 """
 import ctypes as C
+import threading
 
 import torch
 
@@ -94,6 +95,14 @@ SAVE_HIT_MASKS = True
 # With per_pixel_sort and tile lists of at least this many entries on average, depth bounds of the lists are
 # computed (one more pass over the keys) so that the selection can stop before the end of a list.
 EARLY_STOP_MIN_AVG_LIST = 512
+# Binning (count, scan, key emission) in one launch where the library takes the frame (tg_bin_frame_supported);
+# False: tg_bin_setup + tg_build_tile_lists, the route of the double build and of frames with more than 2^21 tiles.
+FUSED_BINNING = True
+
+
+def _as_int32(v):
+    """A uint32 as the int32 it reads back as."""
+    return v - (1 << 32) if v >= (1 << 31) else v
 
 
 def scan_exclusive(counts, out=None, heads=None):
@@ -297,6 +306,86 @@ def build_tile_lists(setup, n_keys, emit_only=False, prepared=None):
     return keys, values, status, offsets
 
 
+# ---- the frame's route: binning in one launch -------------------------------------------------------------
+
+_frame_states = {}  # device index -> dict(frame, epoch): the state tg_bin_frame keeps between calls
+_frame_lock = threading.Lock()
+_FRAME_TAIL = 256  # bytes behind the library's frame state: K and the status word of the binning
+
+
+def bin_frame_supported(vertices, width, height, tile_width, tile_height):
+    """Whether tg_bin_frame takes this frame (float build, at most 65535 tile columns and rows, 2^21 tiles)."""
+    return _bits(vertices) == 32 and bool(_lib.load(32).tg_bin_frame_supported(width, height, tile_width, tile_height))
+
+
+def _next_frame_state(dev, need):
+    """The device's frame state of at least `need` bytes, zeroed when it is made, and the epoch of the call about to
+    use it (they count up by one; a state whose epochs run out is replaced by a fresh one)."""
+    with _frame_lock:
+        st = _frame_states.get(dev.index)
+        if st is None or st["bytes"] < need or st["epoch"] >= 0x3FFFFFF0:
+            size = need + need // 4
+            st = dict(frame=torch.zeros((size + _FRAME_TAIL,), dtype=torch.uint8, device=dev), epoch=0, bytes=size)
+            _frame_states[dev.index] = st
+        st["epoch"] += 1
+        return st["frame"], st["bytes"], st["epoch"]
+
+
+def bin_frame(vertices, indices, width, height, tile_width, tile_height, capacity=None):
+    """Counts, scans and emits without a wait for the host (tg_bin_frame) into buffers for `capacity` keys (default:
+    what the device's last frame needed plus an eighth, or three keys per triangle).
+
+    -> dict(keys, values (emission order, the first min(K, capacity) valid), total_and_status (2,) int32:
+    K and, if a wait expired, `epoch`; capacity, epoch, and the buffers the sort needs)"""
+    _need_cuda(vertices, indices)
+    lib = _lib.load(32)
+    dev = vertices.device
+    M = indices.shape[0]
+    T = num_tiles(width, height, tile_width, tile_height)
+    if capacity is None:
+        hint = _key_count_hint.get(dev.index)
+        capacity = hint + hint // 8 + 1024 if hint is not None else 3 * M + 65536
+    capacity = max(1, min(int(capacity), (1 << 30) - 1))
+    need = int(lib.tg_bin_frame_workspace_bytes(M, capacity, width, height, tile_width, tile_height))
+    frame, frame_bytes, epoch = _next_frame_state(dev, need)
+    pair = frame[frame_bytes:frame_bytes + 8].view(torch.int32)
+    ws_bytes = int(lib.tg_build_frame_lists_workspace_bytes(capacity, T))
+    b = dict(capacity=capacity, epoch=epoch, frame=frame, total_and_status=pair, n_tiles=T, ws_bytes=ws_bytes,
+             keys=torch.empty((capacity,), dtype=torch.int64, device=dev),
+             values=torch.empty((capacity,), dtype=torch.int32, device=dev),
+             keys_alt=torch.empty((capacity,), dtype=torch.int64, device=dev),
+             values_alt=torch.empty((capacity,), dtype=torch.int32, device=dev),
+             offsets=torch.empty((T + 1,), dtype=torch.int32, device=dev),
+             status=torch.empty((1,), dtype=torch.int32, device=dev),
+             ws=torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=dev))
+    # the sort's own histogram route (more than 65536 tiles) clears its workspace itself
+    zero_bytes = ws_bytes if T <= 65536 else 0
+    with _on_device(dev):
+        _lib.check(lib.tg_bin_frame(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
+                                    _ptr(b["keys"]), _ptr(b["values"]), capacity, _ptr(pair), _ptr(frame),
+                                    frame_bytes, epoch, _ptr(b["ws"]), zero_bytes, _ptr(b["status"]), _stream(vertices)),
+                   "tg_bin_frame")
+    return b
+
+
+def build_frame_lists(binned, n_keys):
+    """bin_frame's result + K (at most its capacity) -> (sorted_keys, sorted_ids, status (1,) int32, offsets (T+1,) int32)."""
+    lib = _lib.load(32)
+    b = binned
+    if n_keys > b["capacity"]:
+        raise ValueError(f"{n_keys} keys, buffers for {b['capacity']}")
+    dev = b["keys"].device
+    _key_count_hint[dev.index] = n_keys
+    in_alt = C.c_int(0)
+    with _on_device(dev):
+        _lib.check(lib.tg_build_frame_lists(_ptr(b["frame"]), b["epoch"], n_keys, b["n_tiles"], _ptr(b["keys"]), _ptr(b["values"]),
+                                            _ptr(b["keys_alt"]), _ptr(b["values_alt"]), _ptr(b["offsets"]), _ptr(b["ws"]),
+                                            b["ws_bytes"], _ptr(b["status"]), C.byref(in_alt), _stream(b["keys"])),
+                   "tg_build_frame_lists")
+    keys, values = (b["keys_alt"], b["values_alt"]) if in_alt.value else (b["keys"], b["values"])
+    return keys[:n_keys], values[:n_keys], b["status"], b["offsets"]
+
+
 def cartesian_to_bary(vertices, indices):
     """(M,3,3) cartesian-to-barycentric matrices (reference _C.cartesian_to_bary, render.cu:697-711)."""
     _need_cuda(vertices, indices)
@@ -458,33 +547,37 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
 
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
-        setup = bin_setup(vertices, indices, width, height, tile_width, tile_height)
-        bary_transforms = prepared = None
-        if disable_timing:
-            # K travels to pinned host memory while the device already computes the bary matrices, which do
-            # not depend on it; the host waits for the copy only (with stage timings the reference's order is kept)
-            host = torch.empty((2,), dtype=torch.int32, pin_memory=True)
-            host.copy_(setup["total_and_status"], non_blocking=True)
-            arrived = torch.cuda.Event()
-            arrived.record()
-            bary_transforms = cartesian_to_bary(vertices, indices)
-            prepared = prepare_tile_lists(setup)
-            arrived.synchronize()
+        bary_transforms = None
+        if FUSED_BINNING and bin_frame_supported(vertices, width, height, tile_width, tile_height):
+            # count, scan and emission in one launch into buffers sized by the last frame's K; K and the status word
+            # travel to pinned host memory while the device computes the bary matrices, which do not depend on K
+            binned = bin_frame(vertices, indices, width, height, tile_width, tile_height)
+            while True:
+                host = torch.empty((2,), dtype=torch.int32, pin_memory=True)
+                host.copy_(binned["total_and_status"], non_blocking=True)
+                arrived = torch.cuda.Event()
+                arrived.record()
+                if bary_transforms is None and disable_timing:
+                    bary_transforms = cartesian_to_bary(vertices, indices)
+                arrived.synchronize()
+                K, st = host.tolist()
+                if st == _as_int32(binned["epoch"]):
+                    raise RuntimeError("tg_bin_frame: wait for another workgroup timed out")
+                if K <= binned["capacity"]:
+                    break
+                binned = bin_frame(vertices, indices, width, height, tile_width, tile_height, capacity=K + K // 8)
+            timer.start("sorting")
+            keys, sorted_ids, sort_status, offsets = build_frame_lists(binned, K)
         else:
-            host = setup["total_and_status"].cpu()
-        K, st = host.tolist()  # one conversion: the device waits for the launches that follow
-        if st != 0:
-            raise RuntimeError("tg_bin_setup: look-back wait timed out")
-        if bits == 32 and disable_timing:
-            keys, sorted_ids, sort_status, offsets = build_tile_lists(setup, K, prepared=prepared)
-        else:
-            # the stages apart, so that their times are the reference's (render.cu:733-745); the double build's
-            # depth keys take 64 bits and are sorted in two rounds
+            setup = bin_setup(vertices, indices, width, height, tile_width, tile_height)
+            K, st = setup["total_and_status"].cpu().tolist()
+            if st != 0:
+                raise RuntimeError("tg_bin_setup: look-back wait timed out")
             keys, payload, _, _ = build_tile_lists(setup, K, emit_only=True)
             timer.start("sorting")
             if bits == 32:
                 keys, sorted_ids, sort_status, offsets = sort_tile_lists(keys, payload, T)
-            else:
+            else:  # the double build's depth keys take 64 bits and are sorted in two rounds
                 keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
         status_check = StatusCheck(sort_status)
         _pending_checks.append(status_check)

@@ -58,13 +58,13 @@ ProfileScope::~ProfileScope() {
     if (slot < (int)g_profile_records.size()) (void)hipEventRecord(g_profile_records[slot].stop, stream);
 }
 
-int resident_workgroups(const void *kernel, int threads, int *cache) {
+int resident_workgroups(const void *kernel, int threads, int *cache, size_t dynamic_lds) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
     if (cache[dev] == 0) {
         int per_cu = 0;
         hipDeviceProp_t prop;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess ||
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds) != hipSuccess ||
             hipGetDeviceProperties(&prop, dev) != hipSuccess) {
             (void)hipGetLastError();
             cache[dev] = -1;
@@ -73,6 +73,25 @@ int resident_workgroups(const void *kernel, int threads, int *cache) {
         }
     }
     return cache[dev] > 0 ? cache[dev] : 0;
+}
+
+int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved) {
+    if (bytes <= 64 * 1024) return 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        set_error("%s: no current device", fn);
+        return (int)hipErrorInvalidDevice;
+    }
+    if (bytes <= reserved[dev]) return 0;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("%s: cannot reserve %zu bytes of LDS per workgroup: %s", fn, bytes, hipGetErrorString(e));
+        return (int)e;
+    }
+    reserved[dev] = bytes;
+    return 0;
 }
 
 }  // namespace tg

@@ -1022,13 +1022,11 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
     }
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, pixel_order_threads(kTileThreads));
     const size_t lds = backward_pixel_order_lds_bytes(tl.threads);
-    static size_t lds_reserved = 0;
+    static size_t lds_reserved[3][kMaxDevices] = {{0}};
+    int which = 0;
     for (const void *kernel : {(const void *)backward_pixel_order_kernel<kGradDense>, (const void *)backward_pixel_order_kernel<kGradBlock8>,
-                               (const void *)backward_pixel_order_kernel<kGradStrided>}) {
-        size_t none = 0;
-        if (int e = reserve_lds("tg_render_backward", kernel, lds, lds <= lds_reserved ? &lds_reserved : &none)) return e;
-    }
-    if (lds > lds_reserved) lds_reserved = lds;
+                               (const void *)backward_pixel_order_kernel<kGradStrided>})
+        if (int e = reserve_lds("tg_render_backward", kernel, lds, lds_reserved[which++])) return e;
     TG_LAUNCH_BACKWARD(backward_pixel_order_kernel, tl.grid, dim3(tl.threads), lds);
     return check_launch("backward_pixel_order_kernel");
 #undef TG_LAUNCH_BACKWARD

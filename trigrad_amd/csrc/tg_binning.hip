@@ -34,6 +34,19 @@ __device__ __forceinline__ TriXYZ load_triangle(const real4 *__restrict__ vertic
     return r;
 }
 
+// The three corners of the triangle with the vertex numbers (ia, ib, ic), zeros for a triangle that names a
+// vertex outside [0, n_vertices).
+__device__ __forceinline__ void fetch_corners(const real4 *__restrict__ vertices, int n_vertices, int ia, int ib, int ic, real4 &a,
+                                              real4 &b, real4 &c) {
+    const bool ok = (unsigned)ia < (unsigned)n_vertices && (unsigned)ib < (unsigned)n_vertices && (unsigned)ic < (unsigned)n_vertices;
+    a = b = c = make_real4(0.f, 0.f, 0.f, 0.f);
+    if (ok) {
+        a = vertices[ia];
+        b = vertices[ib];
+        c = vertices[ic];
+    }
+}
+
 __global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                                 const int32_t *__restrict__ indices, int n_triangles, int W,
                                                                 int H, int tw, int th, int tiles_x, int tiles_y,
@@ -48,16 +61,19 @@ __global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const real4 *__r
 // Per-thread polygon storage in LDS, slot-major so that lanes never conflict.
 constexpr int kPolyCap = 8;
 constexpr int kOwnerWindow = 1024;  // triangle offsets staged per workgroup for the owner search
-struct PolyLds {
-    real x[kPolyCap][kBinThreads];
-    real y[kPolyCap][kBinThreads];
+template <int THREADS>
+struct PolyLdsOf {
+    real x[kPolyCap][THREADS];
+    real y[kPolyCap][THREADS];
 };
+using PolyLds = PolyLdsOf<kBinThreads>;
 
 // One Sutherland-Hodgman pass (render.cu:159-189) against nx*x + ny*y - d >= 0, in place.  Returns the new
 // vertex count.  The polygon is read into registers first (the loop over the eight slots is unrolled, so
 // they are plain registers and every distance is computed once); the output goes back to the same LDS slots
 // at its own running index.  When every vertex is inside, the pass reproduces its input and nothing is written.
-__device__ __forceinline__ int clip_pass(PolyLds &lds, int n_in, real nx, real ny, real d) {
+template <typename Poly>
+__device__ __forceinline__ int clip_pass(Poly &lds, int n_in, real nx, real ny, real d) {
     const int tid = threadIdx.x;
     real px[kPolyCap], py[kPolyCap], dist[kPolyCap];
     bool all_in = true;
@@ -217,7 +233,6 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
 constexpr int kRecordReals = TG_RECORD_SCALARS;  // three planes of M x 4: A B C x0 | ax ay bx by | cx cy y0 ny
 static_assert(kRecordReals == 12, "three real4 per triangle");
 constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets
-constexpr int kEmitDigitPasses = 2;  // tile passes whose digits the emission counts (up to 65536 tiles; the caller sees to that)
 constexpr int kStateTotalsWords = kEmitDigitPasses * kRadix * kTotalsStride;
 
 struct FrameState {
@@ -469,6 +484,429 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
     }
 }
 
+// ---- the frame's binning: two launches that leave nothing for the host to do in between ------------------
+//
+// frame_scan_kernel   counts and scans in one pass over the triangles, like bin_setup_kernel, and leaves the same
+//                     records; but every word it shares between workgroups or calls carries the call's epoch, so
+//                     nothing has to be cleared before the launch: a state word of another epoch is "not yet
+//                     written".  The digit totals go to one of two sets in turn (a call counts into one and
+//                     clears the other).  The look-back reads 512 predecessors per round trip.
+// frame_emit_kernel   one workgroup per kEmitChunk key positions.  It reads K from the device, so it is launched
+//                     for the capacity of the key buffers before the host knows K.  Per key it runs only those
+//                     of the four clip passes that can change the polygon, and keys that run the same number of
+//                     passes are put on the same wave.
+// Which passes can be skipped: a pass whose half plane holds every vertex reproduces its input (render.cu:159-189).
+// While the polygon is the triangle itself that is a comparison of the triangle's bounds with the tile edge.  A
+// vertex made by an earlier pass is p0 + t (p1 - p0) with 0 <= t <= 1, which rounding can push past the
+// bounds of p0 and p1 by at most 5 ulps of the largest coordinate; over four passes that stays below 2^-19 of
+// it.  So a pass is left out only when the bounds clear the tile edge by that margin, and is run, with its own
+// test of every vertex, whenever they do not: the polygon is the reference's in every case.
+constexpr int kEmitThreads = 256;
+constexpr int kEmitWaves = kEmitThreads / kWave;
+constexpr int kEmitKeys = 2;  // keys per thread
+constexpr int kEmitChunk = kEmitThreads * kEmitKeys;
+constexpr int kFrameMaxTiles = 1 << 21;  // the reciprocal multiply finds a key's column exactly up to here
+constexpr int kFrameTotalsWords = 2 * kEmitDigitPasses * kRadix;  // two sets: a call counts into one and clears the other
+constexpr int kLookSlots = 8;  // state words a lane of the look-back reads per round trip
+constexpr uint32_t kEpochMask = 0x3fffffffu;
+
+// A workgroup barrier that orders the LDS traffic only.  __syncthreads also waits for every global load and
+// store the wave has in flight, which these kernels' barriers, all between LDS phases, have no use for.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// State word of the scan: bits 63..62 = 1 tile total, 2 inclusive prefix; bits 61..32 = the call's epoch;
+// bits 31..0 = the value.  A word whose epoch is another call's counts as not written.
+__device__ __forceinline__ uint64_t stamped(uint32_t flag, uint32_t epoch, uint32_t value) {
+    return ((uint64_t)flag << 62) | ((uint64_t)(epoch & kEpochMask) << 32) | value;
+}
+__device__ __forceinline__ uint32_t stamp_flag(uint64_t word, uint32_t epoch) {
+    return ((uint32_t)(word >> 32) & kEpochMask) == (epoch & kEpochMask) ? (uint32_t)(word >> 62) : 0u;
+}
+
+// Called by the first wave of the workgroup that owns `tile`: publishes the tile's total, adds up the totals of
+// all earlier tiles (64 * kLookSlots state words per round trip, the nearest inclusive prefix ends the walk),
+// publishes the inclusive prefix and returns the exclusive one.  The last tile writes the grand total.
+__device__ __forceinline__ uint32_t frame_tile_prefix(uint64_t *states, int tile, uint32_t tile_total, int n_tiles, uint32_t epoch,
+                                                      uint32_t *total_and_status) {
+    const int lane = threadIdx.x & (kWave - 1);
+    if (lane == 0) __hip_atomic_store(&states[tile], stamped(tile == 0 ? 2u : 1u, epoch, tile_total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t sum = 0;
+    bool timed_out = false;
+    for (int look = tile - 1; look >= 0; look -= kWave * kLookSlots) {
+        uint64_t word[kLookSlots];
+#pragma unroll
+        for (int k = 0; k < kLookSlots; k++) {
+            const int idx = look - (k * kWave + lane);
+            word[k] = idx >= 0 ? __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : stamped(2u, epoch, 0u);
+        }
+        bool done = false;
+#pragma unroll
+        for (int k = 0; k < kLookSlots; k++) {
+            if (done) continue;  // uniform
+            const int idx = look - (k * kWave + lane);
+            uint32_t spins = 0;
+            while (stamp_flag(word[k], epoch) == 0 && spins < kSpinLimit) {
+                __builtin_amdgcn_s_sleep(1);
+                word[k] = __hip_atomic_load(&states[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                spins++;
+            }
+            const uint32_t flag = stamp_flag(word[k], epoch);
+            if (flag == 0) timed_out = true;
+            const uint64_t inclusive_lanes = __builtin_amdgcn_ballot_w64(flag == 2);
+            const int first = inclusive_lanes ? __builtin_ctzll(inclusive_lanes) : kWave;
+            if (flag != 0 && lane <= first) sum += (uint32_t)word[k];
+            done = inclusive_lanes != 0;
+        }
+        if (done) break;
+    }
+    const uint32_t prefix = wave_sum(sum);
+    if (__builtin_amdgcn_ballot_w64(timed_out) && lane == 0) total_and_status[1] = epoch;
+    if (lane == 0) {
+        if (tile != 0) __hip_atomic_store(&states[tile], stamped(2u, epoch, prefix + tile_total), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tile == n_tiles - 1) total_and_status[0] = prefix + tile_total;
+    }
+    return prefix;
+}
+
+// Like count_tile_digits with short lane loops: a rectangle of up to kLaneRectShort tiles is walked by its lane,
+// larger ones by the whole wave, 64 tiles at a time.
+constexpr uint32_t kLaneRectShort = 6;
+__device__ __forceinline__ void count_tile_digits_short(const Rect &r, uint32_t count, int tiles_x, const PassPlan &plan,
+                                                        uint32_t (*hist)[kRadix]) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int shift0 = plan.shift[0] - 32, shift1 = plan.shift[1] - 32;
+    const uint32_t mask0 = (1u << plan.bits[0]) - 1, mask1 = (1u << plan.bits[1]) - 1;
+    const bool two = plan.passes > 1;
+    if (count > 0 && count <= kLaneRectShort) {
+        int tx = r.x0, ty = r.y0;
+        for (uint32_t i = 0; i < count; i++) {
+            const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
+            atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
+            if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
+            if (++ty > r.y1) { ty = r.y0; tx++; }
+        }
+    }
+    uint64_t large = __builtin_amdgcn_ballot_w64(count > kLaneRectShort);
+    while (large) {
+        const int src = __builtin_ctzll(large);
+        large &= large - 1;
+        const int x0 = __shfl(r.x0, src, kWave), y0 = __shfl(r.y0, src, kWave);
+        const int ny = __shfl(r.y1, src, kWave) - y0 + 1, nx = __shfl(r.x1, src, kWave) - x0 + 1;
+        // lane l takes the tiles l, l + 64, ... of the rectangle in column-major order (column = tile x)
+        int col = lane / ny, row = lane % ny;
+        const int col_step = kWave / ny, row_step = kWave % ny;
+        while (col < nx) {
+            const uint32_t tile = (uint32_t)((y0 + row) * tiles_x + x0 + col);
+            atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
+            if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
+            col += col_step;
+            row += row_step;
+            if (row >= ny) { row -= ny; col++; }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kScanThreads) void frame_scan_kernel(const real4 *__restrict__ vertices, int n_vertices,
+                                                                  const int32_t *__restrict__ indices, int n_triangles, int W, int H,
+                                                                  int tw, int th, int tiles_x, int tiles_y, uint32_t epoch,
+                                                                  uint32_t *__restrict__ tri_offsets, real4 *__restrict__ records,
+                                                                  uint32_t *total_and_status, uint32_t *ticket, uint64_t *states,
+                                                                  int n_scan_tiles, uint32_t head_capacity, uint32_t *__restrict__ heads,
+                                                                  PassPlan plan, uint32_t *totals, uint32_t *totals_next,
+                                                                  real *__restrict__ edges, uint32_t *zero, size_t zero_words,
+                                                                  uint32_t *clear_word) {
+    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_wave_total[kScanThreads / kWave];
+    __shared__ uint32_t s_tile_prefix;
+    __shared__ uint32_t s_count[kScanTile];
+    __shared__ uint32_t s_hist[kEmitDigitPasses][kRadix];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    if (totals && tid < kRadix)
+        for (int p = 0; p < kEmitDigitPasses; p++) s_hist[p][tid] = 0;
+    if (tid == 0) {
+        uint32_t mine = blockIdx.x;  // no ticket: the whole grid is resident
+        if (ticket) {
+            mine = atomicAdd(ticket, 1u);
+            if (mine == (uint32_t)n_scan_tiles - 1) atomicExch(ticket, 0u);  // all tickets are out: ready for the next call
+        }
+        s_tile = mine;
+    }
+    // side jobs: what the sort wants cleared, the other set of digit totals, the NDC edges of the tile columns and rows
+    for (size_t i = (size_t)blockIdx.x * kScanThreads + tid; i < zero_words; i += (size_t)gridDim.x * kScanThreads) zero[i] = 0;
+    if (blockIdx.x == 0) {
+        if (totals_next && tid < kEmitDigitPasses * kRadix) totals_next[tid] = 0;
+        if (clear_word && tid == 0) *clear_word = 0;
+        // render.cu:243-246: the edges of tile column tx are entries tx and tx + 1
+        for (int i = tid; i <= tiles_x; i += kScanThreads) edges[i] = (real)(i * tw) / (real)W * 2.0f - 1.0f;
+        for (int i = tid; i <= tiles_y; i += kScanThreads) edges[tiles_x + 1 + i] = (real)(i * th) / (real)H * 2.0f - 1.0f;
+    }
+    lds_barrier();
+    const int tile = (int)s_tile;
+    const int64_t base = (int64_t)tile * kScanTile + (int64_t)tid * 4;
+
+    // Triangle by triangle across the lanes (neighbouring lanes take neighbouring triangles, so the index
+    // loads and the record stores of a wave are contiguous); the counts then change hands through LDS so that
+    // every thread scans four consecutive ones.
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int64_t t = (int64_t)tile * kScanTile + k * kScanThreads + tid;
+        uint32_t count = 0;
+        Rect rect = {0, -1, 0, -1};
+        if (t < n_triangles) {
+            const TriXYZ p = load_triangle(vertices, n_vertices, indices, (int)t);
+            const Rect r = tile_rect(p.ax, p.ay, p.bx, p.by, p.cx, p.cy, W, H, tw, th, tiles_x, tiles_y);
+            count = rect_count(r);
+            // render.cu:140-152 compute_plane
+            const real det = p.ax * (p.by - p.cy) + p.bx * (p.cy - p.ay) + p.cx * (p.ay - p.by);
+            const real id = (real)(1.0 / (double)det);
+            const real A = (p.az * (p.by - p.cy) + p.bz * (p.cy - p.ay) + p.cz * (p.ay - p.by)) * id;
+            const real B = (p.ax * (p.bz - p.cz) + p.bx * (p.cz - p.az) + p.cx * (p.az - p.bz)) * id;
+            const real C = (p.ax * (p.by * p.cz - p.cy * p.bz) + p.bx * (p.cy * p.az - p.ay * p.cz) + p.cx * (p.ay * p.bz - p.by * p.az)) * id;
+            records[t] = make_real4(A, B, C, int_in_real(r.x0));
+            records[(int64_t)n_triangles + t] = make_real4(p.ax, p.ay, p.bx, p.by);
+            records[2 * (int64_t)n_triangles + t] = make_real4(p.cx, p.cy, int_in_real(r.y0), int_in_real(r.y1 - r.y0 + 1));
+            rect = r;
+        }
+        s_count[k * kScanThreads + tid] = count;
+        if (totals) count_tile_digits_short(rect, count, tiles_x, plan, s_hist);
+    }
+    lds_barrier();
+    if (totals && tid < kRadix)
+        for (int p = 0; p < plan.passes; p++) {
+            const uint32_t c = s_hist[p][tid];
+            if (c) atomicAdd(&totals[p * kRadix + tid], c);
+        }
+    uint32_t x[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) x[k] = s_count[tid * 4 + k];
+    const uint32_t thread_sum = x[0] + x[1] + x[2] + x[3];
+    const uint32_t incl = wave_inclusive_scan_u32(thread_sum);
+    if (lane == kWave - 1) s_wave_total[wave] = incl;
+    lds_barrier();
+    if (wave == 0) {
+        uint32_t wt = (lane < kScanThreads / kWave) ? s_wave_total[lane] : 0u;
+        uint32_t wincl = wave_inclusive_scan_u32(wt);
+        uint32_t tile_total = (uint32_t)__builtin_amdgcn_readlane((int)wincl, kScanThreads / kWave - 1);
+        if (lane < kScanThreads / kWave) s_wave_total[lane] = wincl - wt;  // exclusive wave offsets
+        const uint32_t prefix = frame_tile_prefix(states, tile, tile_total, n_scan_tiles, epoch, total_and_status);
+        if (lane == 0) s_tile_prefix = prefix;
+    }
+    lds_barrier();
+    uint32_t run = s_tile_prefix + s_wave_total[wave] + (incl - thread_sum);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int64_t t = base + k;
+        if (t >= n_triangles) break;
+        tri_offsets[t] = run;
+        if (x[k] != 0) {
+            // triangle t owns the key positions [run, run + x): note for every multiple of kEmitChunk who owns it
+            const uint32_t first = (run + kEmitChunk - 1) / kEmitChunk, last = (run + x[k] - 1) / kEmitChunk;
+            for (uint32_t h = first; h <= last && h < head_capacity; h++) heads[h] = (uint32_t)t;
+        }
+        run += x[k];
+    }
+}
+
+#ifndef TG_DOUBLE_PRECISION
+__device__ __forceinline__ uint32_t dpp_max_u32_step(uint32_t v, uint32_t o) { return o > v ? o : v; }
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+    return dpp_max_u32_step(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kCtrl, kRowMask, 0xf, false));
+}
+__device__ __forceinline__ uint32_t wave_inclusive_max_u32(uint32_t v) {
+    v = dpp_max_u32<0x111, 0xf>(v);
+    v = dpp_max_u32<0x112, 0xf>(v);
+    v = dpp_max_u32<0x114, 0xf>(v);
+    v = dpp_max_u32<0x118, 0xf>(v);
+    v = dpp_max_u32<0x142, 0xa>(v);
+    v = dpp_max_u32<0x143, 0xc>(v);
+    return v;
+}
+
+struct EmitLds {
+    PolyLdsOf<kEmitThreads> poly;  // the polygon of the key a thread clips
+    uint32_t owner[kEmitChunk];    // per key position of the chunk: first the marks of the triangles' first keys, then the owners
+    uint16_t queue[kEmitChunk];    // the chunk's keys that need clipping, those with the most passes first
+    uint32_t wave_owner[kEmitWaves];
+    uint32_t bucket[4];            // keys of the chunk with 4, 3, 2, 1 passes to run
+};
+
+// What a key needs from its triangle's record and its position in the tile rectangle.
+struct FrameKey {
+    real A, B, C, ax, ay, bx, by, cx, cy;
+    real xmin, xmax, ymin, ymax;  // render.cu:243-246 tile rectangle in NDC
+    uint32_t tile_id;
+};
+__device__ __forceinline__ FrameKey frame_key(const real4 *__restrict__ records, int n_triangles, int t, uint32_t local,
+                                              const real *__restrict__ edges, int tiles_x) {
+    const real4 r0 = records[t], r1 = records[(int64_t)n_triangles + t], r2 = records[2 * (int64_t)n_triangles + t];
+    FrameKey k;
+    k.A = r0.x; k.B = r0.y; k.C = r0.z;
+    k.ax = r1.x; k.ay = r1.y; k.bx = r1.z; k.by = r1.w; k.cx = r2.x; k.cy = r2.y;
+    const uint32_t ny = (uint32_t)int_of_real(r2.w);
+    // column = local / ny, row = local % ny (tile x outer, tile y inner, render.cu:235-236): the reciprocal
+    // multiply is off by at most one for local < 2^21
+    uint32_t col = (uint32_t)((float)local * __builtin_amdgcn_rcpf((float)ny));
+    int row = (int)local - (int)(col * ny);
+    if (row < 0) { col--; row += (int)ny; } else if (row >= (int)ny) { col++; row -= (int)ny; }
+    const int tx = int_of_real(r0.w) + (int)col, ty = int_of_real(r2.z) + row;
+    k.xmin = edges[tx]; k.xmax = edges[tx + 1];  // a few hundred scalars that every key reads: they stay in cache
+    k.ymin = edges[tiles_x + 1 + ty]; k.ymax = edges[tiles_x + 2 + ty];
+    k.tile_id = (uint32_t)(ty * tiles_x + tx);
+    return k;
+}
+// The clip passes that may change the key's polygon (bit b: pass b of render.cu:254-257), see above.
+__device__ __forceinline__ uint32_t frame_key_passes(const FrameKey &k) {
+    const real lo_x = min3(k.ax, k.bx, k.cx), hi_x = max3(k.ax, k.bx, k.cx);
+    const real lo_y = min3(k.ay, k.by, k.cy), hi_y = max3(k.ay, k.by, k.cy);
+    const real x_abs = abs_real(lo_x) > abs_real(hi_x) ? abs_real(lo_x) : abs_real(hi_x);
+    const real y_abs = abs_real(lo_y) > abs_real(hi_y) ? abs_real(lo_y) : abs_real(hi_y);
+    const real slack_x = x_abs * 1.9073486328125e-06f + 1e-37f, slack_y = y_abs * 1.9073486328125e-06f + 1e-37f;  // 2^-19
+    uint32_t todo = 0;
+    if (!(lo_x - slack_x >= k.xmin)) todo |= 1u;
+    if (!(hi_x + slack_x <= k.xmax)) todo |= 2u;
+    if (!(lo_y - slack_y >= k.ymin)) todo |= 4u;
+    if (!(hi_y + slack_y <= k.ymax)) todo |= 8u;
+    return todo;
+}
+
+__global__ __launch_bounds__(kEmitThreads) void frame_emit_kernel(const real4 *__restrict__ records, const uint32_t *__restrict__ tri_offsets,
+                                                                  int n_triangles, const uint32_t *__restrict__ total_and_status,
+                                                                  uint32_t key_capacity, const uint32_t *__restrict__ heads,
+                                                                  uint32_t head_capacity, const real *__restrict__ edges, int tiles_x,
+                                                                  uint64_t *__restrict__ keys, uint32_t *__restrict__ payload) {
+    __shared__ EmitLds L;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const uint32_t total = total_and_status[0];
+    const uint32_t n_keys = total < key_capacity ? total : key_capacity;  // keys beyond the buffers are left out
+    const uint32_t k0 = blockIdx.x * (uint32_t)kEmitChunk;
+    if (k0 >= n_keys) return;
+    // The owners of the chunk's keys lie between the owner of its first key and the owner of the next chunk's
+    // first key; the scan noted both (otherwise two uniform binary searches find them).
+    int t_first, t_last;
+    if (blockIdx.x < head_capacity) {
+        t_first = (int)heads[blockIdx.x];
+        t_last = (k0 + kEmitChunk < total && blockIdx.x + 1 < head_capacity) ? (int)heads[blockIdx.x + 1] : n_triangles - 1;
+    } else {
+        const uint32_t k_last = (k0 + kEmitChunk <= n_keys ? k0 + kEmitChunk : n_keys) - 1;
+        t_first = owner_of_key(tri_offsets, n_triangles, k0);
+        t_last = owner_of_key(tri_offsets, n_triangles, k_last);
+    }
+    const int span = t_last - t_first + 1;
+    L.owner[tid] = 0;
+    L.owner[kEmitThreads + tid] = 0;
+    if (tid < 4) L.bucket[tid] = 0;
+    lds_barrier();
+    // every triangle of the span marks the position of its first key in the chunk with its number (+ 1); of
+    // several triangles at one position (all but the last own no key) the last counts
+    for (int i = tid; i < span; i += kEmitThreads) {
+        const uint32_t off = tri_offsets[t_first + i];
+        if (off < k0 + kEmitChunk) atomicMax(&L.owner[off > k0 ? off - k0 : 0u], (uint32_t)i + 1u);
+    }
+    lds_barrier();
+    // a running maximum over the marks gives every key position its triangle
+    {
+        uint32_t m0 = L.owner[2 * tid], m1 = L.owner[2 * tid + 1];
+        m1 = m1 > m0 ? m1 : m0;
+        const uint32_t wmax = wave_inclusive_max_u32(m1);
+        if (lane == kWave - 1) L.wave_owner[wave] = wmax;
+        uint32_t before = (uint32_t)__shfl_up((int)wmax, 1, kWave);
+        if (lane == 0) before = 0;
+        lds_barrier();
+        for (int w = 0; w < wave; w++) before = L.wave_owner[w] > before ? L.wave_owner[w] : before;
+        L.owner[2 * tid] = m0 > before ? m0 : before;
+        L.owner[2 * tid + 1] = m1 > before ? m1 : before;
+    }
+    lds_barrier();
+
+    // every key of the chunk, neighbouring keys on neighbouring lanes: its tile and the passes it needs.  A key
+    // that needs none is done here (its polygon is the triangle, render.cu:262-267); the others queue up by
+    // their number of passes.
+    uint32_t entry[kEmitKeys], slot[kEmitKeys];
+#pragma unroll
+    for (int k = 0; k < kEmitKeys; k++) {
+        const uint32_t in_chunk = (uint32_t)k * kEmitThreads + tid, at = k0 + in_chunk;
+        uint32_t e = 0, at_slot = 0;
+        if (at < n_keys) {
+            const uint32_t m = L.owner[in_chunk];
+            const int t = t_first + (m ? (int)m - 1 : 0);  // every key position has a mark at or before it
+            const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x);
+            const uint32_t todo = frame_key_passes(key);
+            if (todo == 0) {
+                real md = std::numeric_limits<real>::max();
+                real pd = key.A * key.ax + key.B * key.ay + key.C;  // render.cu:154-157
+                md = (pd < md) ? pd : md;
+                pd = key.A * key.bx + key.B * key.by + key.C;
+                md = (pd < md) ? pd : md;
+                pd = key.A * key.cx + key.B * key.cy + key.C;
+                md = (pd < md) ? pd : md;
+                keys[at] = ((uint64_t)key.tile_id << 32) | orderable_bits(md);
+                payload[at] = (uint32_t)t;
+            } else {
+                e = 0x8000u | todo | (in_chunk << 4);
+                at_slot = atomicAdd(&L.bucket[4 - __builtin_popcount(todo)], 1u);
+            }
+        }
+        entry[k] = e;
+        slot[k] = at_slot;
+    }
+    lds_barrier();
+    const uint32_t b4 = L.bucket[0], b3 = L.bucket[1], b2 = L.bucket[2], b1 = L.bucket[3];
+    const uint32_t queued = b4 + b3 + b2 + b1;
+#pragma unroll
+    for (int k = 0; k < kEmitKeys; k++)
+        if (entry[k]) {
+            const int passes = __builtin_popcount(entry[k] & 15u);
+            const uint32_t first = passes == 4 ? 0u : passes == 3 ? b4 : passes == 2 ? b4 + b3 : b4 + b3 + b2;
+            L.queue[first + slot[k]] = (uint16_t)entry[k];
+        }
+    lds_barrier();
+    // the queue, 64 keys at a time per wave: neighbours run the same number of passes
+#pragma unroll 1
+    for (uint32_t q = (uint32_t)wave * kWave; q < queued; q += kEmitThreads) {
+        if (q + lane >= queued) continue;
+        const uint32_t e = L.queue[q + lane];
+        const uint32_t in_chunk = (e >> 4) & (kEmitChunk - 1), at = k0 + in_chunk;
+        uint32_t todo = e & 15u;
+        const uint32_t m = L.owner[in_chunk];
+        const int t = t_first + (m ? (int)m - 1 : 0);
+        const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x);
+        L.poly.x[0][tid] = key.ax; L.poly.y[0][tid] = key.ay;
+        L.poly.x[1][tid] = key.bx; L.poly.y[1][tid] = key.by;
+        L.poly.x[2][tid] = key.cx; L.poly.y[2][tid] = key.cy;
+        int n = 3;
+        while (todo) {
+            const uint32_t b = (uint32_t)__builtin_ctz(todo);
+            todo &= todo - 1;
+            const real nx = b == 0 ? 1.0f : (b == 1 ? -1.0f : 0.0f), nyv = b == 2 ? 1.0f : (b == 3 ? -1.0f : 0.0f);
+            const real d = b == 0 ? key.xmin : (b == 1 ? -key.xmax : (b == 2 ? key.ymin : -key.ymax));
+            n = clip_pass(L.poly, n, nx, nyv, d);
+            if (n <= 0) todo = 0;
+        }
+        real depth = kFarKey;  // render.cu:259
+        if (n > 0) {
+            real md = std::numeric_limits<real>::max();
+            for (int i = 0; i < n; i++) {
+                const real pd = key.A * L.poly.x[i][tid] + key.B * L.poly.y[i][tid] + key.C;  // render.cu:154-157
+                md = (pd < md) ? pd : md;
+            }
+            depth = md;
+        }
+        keys[at] = ((uint64_t)key.tile_id << 32) | orderable_bits(depth);
+        payload[at] = (uint32_t)t;
+    }
+}
+#endif  // !TG_DOUBLE_PRECISION
+
+
 // Lower bounds of the per-pixel depths (render.cu:404: interpolate3 of the vertex z with the vertex w
 // as weights) of the rest of every tile list, per batch of kBoundSpan entries.  With positive finite
 // weights the interpolated depth is a convex combination of the three vertex depths, so it cannot lie
@@ -693,11 +1131,110 @@ extern "C" int tg_bin_setup(const real *vertices, int32_t n_vertices, const int3
     // the digits of the sort's tile passes are counted here, where every triangle's tile rectangle is at hand
     // (the double build sorts differently, and more than 65536 tiles take a third pass: no counts then)
     const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
-    const bool count_digits = sizeof(real) == 4 && plan.passes <= kEmitDigitPasses;
+    const bool count_digits = binning_counts_digits(tiles_x * tiles_y);
     TG_LAUNCH(bin_setup_kernel, dim3(n_scan_tiles), dim3(kScanThreads), 0, s, (const real4 *)vertices, n_vertices, indices, n_triangles,
               width, height, tile_w, tile_h, tiles_x, tiles_y, tri_offsets, (real4 *)records, total_and_status, total_and_status + 1,
               ticket, f.states, n_scan_tiles, head_capacity, heads, plan, count_digits ? f.totals : (uint32_t *)nullptr);
     return check_launch("bin_setup_kernel");
+}
+
+// ---- the frame's binning in one call ----
+namespace tg {
+struct FusedFrame {
+    uint32_t *totals;  // two sets of kEmitDigitPasses * kRadix digit totals
+    uint32_t *ticket;
+    uint64_t *states;  // one word per kScanTile triangles
+    real *edges;       // tiles_x + 1 column edges, then tiles_y + 1 row edges
+    uint32_t *heads;   // the owner of every kEmitChunk-th key position
+    uint32_t *tri_offsets;
+    real4 *records;
+    uint32_t head_capacity;
+    size_t bytes;
+};
+static FusedFrame fused_frame(void *base, int64_t n_triangles, int64_t key_capacity, int tiles_x, int tiles_y) {
+    FusedFrame f;
+    char *p = (char *)base;
+    size_t o = 0;
+    const auto take = [&](size_t bytes) { char *at = p + o; o = (o + bytes + 255) & ~(size_t)255; return at; };
+    f.totals = (uint32_t *)take((size_t)kFrameTotalsWords * 4);
+    f.ticket = (uint32_t *)take(4);
+    f.states = (uint64_t *)take((size_t)(ceil_div64(n_triangles, kScanTile) + 1) * 8);
+    f.edges = (real *)take((size_t)(tiles_x + tiles_y + 2) * sizeof(real));
+    f.head_capacity = (uint32_t)(key_capacity / kEmitChunk + 2);
+    f.heads = (uint32_t *)take((size_t)f.head_capacity * 4);
+    f.tri_offsets = (uint32_t *)take((size_t)n_triangles * 4);
+    f.records = (real4 *)take((size_t)n_triangles * kRecordReals * sizeof(real));
+    f.bytes = o;
+    return f;
+}
+uint32_t *fused_frame_totals(void *frame, uint32_t epoch) { return (uint32_t *)frame + (epoch & 1u) * (kEmitDigitPasses * kRadix); }
+
+__global__ void bin_frame_empty_kernel(uint32_t *total_and_status, uint32_t *clear_word) {
+    if (threadIdx.x == 0) {
+        total_and_status[0] = 0;
+        if (clear_word) *clear_word = 0;
+    }
+}
+}  // namespace tg
+
+extern "C" int tg_bin_frame_supported(int width, int height, int tile_w, int tile_h) {
+    if (sizeof(real) != 4 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0) return 0;
+    const int64_t tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
+    return tiles_x * tiles_y <= kFrameMaxTiles;
+}
+
+extern "C" size_t tg_bin_frame_workspace_bytes(int32_t n_triangles, int64_t key_capacity, int width, int height, int tile_w, int tile_h) {
+    if (n_triangles < 0 || key_capacity < 0 || width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0) return 0;
+    return fused_frame(nullptr, n_triangles, key_capacity, ceil_div(width, tile_w), ceil_div(height, tile_h)).bytes;
+}
+
+extern "C" int tg_bin_frame(const real *vertices, int32_t n_vertices, const int32_t *indices, int32_t n_triangles, int width,
+                            int height, int tile_w, int tile_h, uint64_t *keys, uint32_t *values, int64_t key_capacity,
+                            uint32_t *total_and_status, void *frame, size_t frame_bytes, uint32_t epoch, void *zero,
+                            size_t zero_bytes, uint32_t *clear_word, void *stream) {
+#ifdef TG_DOUBLE_PRECISION
+    set_error("tg_bin_frame: the double build's depth keys take all 64 key bits; use tg_bin_setup and tg_build_tile_lists");
+    return TG_E_ARG;
+#else
+    if (int e = check_geometry("tg_bin_frame", vertices, n_vertices, indices, n_triangles, width, height, tile_w, tile_h)) return e;
+    if (!tg_bin_frame_supported(width, height, tile_w, tile_h)) {
+        set_error("tg_bin_frame: more than %d tiles; use tg_bin_setup and tg_build_tile_lists", kFrameMaxTiles);
+        return TG_E_ARG;
+    }
+    if (!total_and_status || !frame || ((uintptr_t)frame & 255) || key_capacity < 0 || key_capacity > kSortMaxN ||
+        (key_capacity > 0 && (!keys || !values)) || ((uintptr_t)keys & 7) || ((uintptr_t)zero & 3) || (zero_bytes & 3) ||
+        (zero_bytes > 0 && !zero) || (epoch & kEpochMask) == 0) {
+        set_error("tg_bin_frame: null or misaligned pointer, key_capacity outside [0, 2^30), or an epoch whose low 30 bits are 0");
+        return TG_E_ARG;
+    }
+    const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
+    const FusedFrame f = fused_frame(frame, n_triangles, key_capacity, tiles_x, tiles_y);
+    if (frame_bytes < f.bytes) {
+        set_error("tg_bin_frame: frame state of %zu bytes, need %zu", frame_bytes, f.bytes);
+        return TG_E_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (n_triangles == 0) {
+        TG_LAUNCH(bin_frame_empty_kernel, dim3(1), dim3(64), 0, s, total_and_status, clear_word);
+        return check_launch("bin_frame_empty_kernel");
+    }
+    const int n_scan_tiles = (int)ceil_div64(n_triangles, kScanTile);
+    static int resident_cache[kMaxDevices] = {0};
+    uint32_t *ticket = f.ticket;
+    if (n_scan_tiles <= resident_workgroups((const void *)frame_scan_kernel, kScanThreads, resident_cache)) ticket = nullptr;
+    const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
+    const bool count_digits = binning_counts_digits(tiles_x * tiles_y);
+    TG_LAUNCH(frame_scan_kernel, dim3(n_scan_tiles), dim3(kScanThreads), 0, s, (const real4 *)vertices, n_vertices, indices, n_triangles,
+              width, height, tile_w, tile_h, tiles_x, tiles_y, epoch, f.tri_offsets, f.records, total_and_status, ticket, f.states,
+              n_scan_tiles, f.head_capacity, f.heads, plan, count_digits ? fused_frame_totals(frame, epoch) : (uint32_t *)nullptr,
+              fused_frame_totals(frame, epoch + 1), f.edges, (uint32_t *)zero, zero_bytes / 4, clear_word);
+    if (int e = check_launch("frame_scan_kernel")) return e;
+    if (key_capacity == 0) return 0;
+    // for every key position the buffers hold: the kernel reads K and the workgroups behind it leave at once
+    TG_LAUNCH(frame_emit_kernel, dim3((unsigned)ceil_div64(key_capacity, kEmitChunk)), dim3(kEmitThreads), 0, s, f.records, f.tri_offsets,
+              n_triangles, total_and_status, (uint32_t)key_capacity, f.heads, f.head_capacity, f.edges, tiles_x, keys, values);
+    return check_launch("frame_emit_kernel");
+#endif
 }
 
 namespace tg {

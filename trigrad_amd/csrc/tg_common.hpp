@@ -62,8 +62,11 @@ struct ProfileScope {
 // (0 if unknown).  A grid that is no larger needs no ticket to number its
 // workgroups for a look-back chain: every workgroup is started without waiting
 // for another to finish, so waiting on lower-numbered ones cannot deadlock.
-int resident_workgroups(const void *kernel, int threads, int *cache /* [kMaxDevices] */);
+int resident_workgroups(const void *kernel, int threads, int *cache /* [kMaxDevices] */, size_t dynamic_lds = 0);
 constexpr int kMaxDevices = 64;
+// Dynamic LDS beyond 64 KB has to be enabled per kernel and device once; `reserved` ([kMaxDevices], zero at
+// first) remembers per device what the kernel has been given.
+int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

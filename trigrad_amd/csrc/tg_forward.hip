@@ -361,18 +361,6 @@ size_t pixel_order_lds_bytes(int n_threads, int staged_entries, size_t position_
     return sizeof(DepthRecord) * staged_entries + (size_t)kLayers * n_threads * (sizeof(real) + position_bytes);
 }
 
-// Dynamic LDS beyond 64 KB has to be enabled per kernel once.
-int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved) {
-    if (bytes <= 64 * 1024 || bytes <= *reserved) return 0;
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) {
-        set_error("%s: cannot reserve %zu bytes of LDS per workgroup: %s", fn, bytes, hipGetErrorString(e));
-        return (int)e;
-    }
-    *reserved = bytes;
-    return 0;
-}
-
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers) {
     if (width <= 0 || height <= 0 || tile_w <= 0 || tile_h <= 0 || tile_w * tile_h > kMaxTilePixels) {
         set_error("%s: image size must be positive and tile_w*tile_h in [1, %d]", fn, kMaxTilePixels);
@@ -438,21 +426,21 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
     const size_t lds = pixel_order_lds_bytes(n_threads, kSelectBatch);
     // Depth bounds make the batches jump in steps of kSelectBatch, so they go with the int positions.
     const bool split = !a.batch_bounds && n_threads >= kSelectBatchShort;
-    static size_t lds_reserved = 0, lds_reserved_long = 0;
+    static size_t lds_reserved[kMaxDevices] = {0}, lds_reserved_long[kMaxDevices] = {0};
     if (!split) {
-        if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatch, int>, lds, &lds_reserved)) return e;
+        if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatch, int>, lds, lds_reserved)) return e;
         TG_LAUNCH_AS("forward_pixel_order_kernel", (forward_pixel_order_kernel<kSelectBatch, int>), grid, dim3(n_threads), lds, s, a, o);
         return check_launch("forward_pixel_order_kernel");
     }
     const size_t lds_short = pixel_order_lds_bytes(n_threads, kSelectBatchShort, sizeof(uint16_t));
-    static size_t lds_reserved_short = 0;
+    static size_t lds_reserved_short[kMaxDevices] = {0};
     if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_kernel<kSelectBatchShort, uint16_t>, lds_short,
-                            &lds_reserved_short))
+                            lds_reserved_short))
         return e;
     TG_LAUNCH_AS("forward_pixel_order_kernel", (forward_pixel_order_kernel<kSelectBatchShort, uint16_t>), grid, dim3(n_threads),
                  lds_short, s, a, o);
     if (int e = check_launch("forward_pixel_order_kernel")) return e;
-    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_long_lists_kernel, lds, &lds_reserved_long)) return e;
+    if (int e = reserve_lds("tg_render_forward", (const void *)forward_pixel_order_long_lists_kernel, lds, lds_reserved_long)) return e;
     const int tiles = (int)(grid.x * grid.y);
     TG_LAUNCH(forward_pixel_order_long_lists_kernel, dim3(min(tiles, kLongListGroups), 1, grid.z), dim3(n_threads), lds, s, a, o,
               (int)grid.x, (int)grid.y);

@@ -217,7 +217,6 @@ TileLaunch tile_launch(int width, int height, int tile_w, int tile_h, int max_th
 int pixel_order_threads(int preferred);
 size_t pixel_order_lds_bytes(int n_threads, int staged_entries, size_t position_bytes = sizeof(int));
 int check_raster_args(const char *fn, int width, int height, int tile_w, int tile_h, int max_layers);
-int reserve_lds(const char *fn, const void *kernel, size_t bytes, size_t *reserved);
 
 // ---- per-wave culling ------------------------------------------------------------------
 // A wave owns 64 pixels of the tile.  Before its lanes test a list entry, the

@@ -945,14 +945,11 @@ static size_t build_lookback_bytes(int64_t n_keys, int n_tiles) {
     return (size_t)plan.passes * lookback_words_per_pass(n_sort_tiles > 0 ? n_sort_tiles : 1) * 4;
 }
 
-// The emission counts the digits of at most this many tile passes (65536 tiles); with more tiles the sort
-// makes its own histogram.
-constexpr int kEmitDigitPasses = 2;
-
+constexpr size_t kFrameSortHeadBytes = 256;  // tg_build_frame_lists: the sweeps' tickets in front of the look-back words
 extern "C" size_t tg_build_tile_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
     if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0) return 0;
-    if (tile_pass_plan(n_tiles).passes > kEmitDigitPasses) return tg_tile_list_sort_workspace_bytes(n_keys, n_tiles);
-    return build_lookback_bytes(n_keys, n_tiles);
+    if (!binning_counts_digits(n_tiles)) return tg_tile_list_sort_workspace_bytes(n_keys, n_tiles);
+    return build_lookback_bytes(n_keys, n_tiles) + kFrameSortHeadBytes;
 }
 
 extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offsets, int32_t n_triangles, int64_t n_keys,
@@ -988,7 +985,7 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
         set_error("tg_build_tile_lists: the double build's depth keys take all 64 key bits; emit only, then sort by depth and by tile");
         return TG_E_ARG;
     }
-    if (tile_pass_plan(n_tiles).passes > kEmitDigitPasses) {
+    if (!binning_counts_digits(n_tiles)) {
         if (int e = launch_emit_records("bin_emit_records_kernel", records, tri_offsets, n_triangles, n_keys, head_capacity, heads,
                                         frame, width, height, tile_w, tile_h, keys, values, nullptr, 0, status, s))
             return e;
@@ -1011,6 +1008,49 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     uint32_t *tickets = frame_tickets(frame);
     if (int e = run_sweeps("tg_build_tile_lists", plan, (int)ceil_div64(n_keys, kSortTile), frame_totals(frame, n_triangles, tiles_x, tiles_y),
                            1, lookback, tickets + 8, keys, values, keys_alt, values_alt, n_keys, status, s))
+        return e;
+    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
+    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
+    *result_in_alt = (plan.passes & 1);
+    return ranges_and_segments(k, v, k_other, v_other, n_keys, n_tiles, offsets, s);
+}
+
+// ---- the tile lists of a frame whose keys tg_bin_frame emitted ------------------------------------------
+extern "C" size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
+    return tg_build_tile_lists_workspace_bytes(n_keys, n_tiles);
+}
+
+extern "C" int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int n_tiles, uint64_t *keys, uint32_t *values,
+                                    uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
+                                    size_t workspace_bytes, uint32_t *status, int *result_in_alt, void *stream) {
+    if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0 || !frame || !result_in_alt || !offsets) {
+        set_error("tg_build_frame_lists: n_keys must be in [0, 2^30), n_tiles positive, frame state, offsets and result_in_alt given");
+        return TG_E_ARG;
+    }
+    *result_in_alt = 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (sizeof(real) != 4) {
+        set_error("tg_build_frame_lists: float build only");
+        return TG_E_ARG;
+    }
+    if (n_keys == 0) {
+        TG_LAUNCH(tile_ranges_kernel, dim3(1), dim3(kSortThreads), 0, s, keys, n_keys, n_tiles, offsets);
+        return check_launch("tile_ranges_kernel");
+    }
+    if (!binning_counts_digits(n_tiles))
+        return sort_tile_lists_run("tg_build_frame_lists", keys, values, keys_alt, values_alt, n_keys, n_tiles, offsets, workspace,
+                                   workspace_bytes, status, result_in_alt, s);
+    if (int e = check_sort_buffers("tg_build_frame_lists", keys, values, keys_alt, values_alt, workspace)) return e;
+    const size_t need = build_lookback_bytes(n_keys, n_tiles) + kFrameSortHeadBytes;
+    if (workspace_bytes < need) {
+        set_error("tg_build_frame_lists: workspace of %zu bytes, need %zu", workspace_bytes, need);
+        return TG_E_WORKSPACE;
+    }
+    uint32_t *tickets = (uint32_t *)workspace;
+    uint32_t *lookback = (uint32_t *)((char *)workspace + kFrameSortHeadBytes);
+    const PassPlan plan = tile_pass_plan(n_tiles);
+    if (int e = run_sweeps("tg_build_frame_lists", plan, (int)ceil_div64(n_keys, kSortTile), fused_frame_totals(frame, epoch), 1, lookback,
+                           tickets, keys, values, keys_alt, values_alt, n_keys, status, s))
         return e;
     uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
     uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;

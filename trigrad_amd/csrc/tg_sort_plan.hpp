@@ -89,6 +89,11 @@ inline int tile_bits_of(int n_tiles) {
 }
 inline PassPlan tile_pass_plan(int n_tiles) { return plan_passes(32, 32 + tile_bits_of(n_tiles)); }
 
+// The binning counts the digits of at most this many tile passes (65536 tiles) for the sort; with more tiles,
+// and in the double build (whose depth keys take all 64 bits), the sort makes its own histogram.
+constexpr int kEmitDigitPasses = 2;
+inline bool binning_counts_digits(int n_tiles) { return sizeof(real) == 4 && tile_pass_plan(n_tiles).passes <= kEmitDigitPasses; }
+
 
 // Key emission from the triangle records of the frame's binning (tg_binning.hip); it clears zero_words words
 // at `zero` and *clear_word.  The frame state's digit totals come from the binning kernel.
@@ -98,5 +103,7 @@ int launch_emit_records(const char *fn, const real *records, const uint32_t *tri
                         hipStream_t s);
 uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y);
 uint32_t *frame_tickets(void *frame);
+// The digit totals that tg_bin_frame(frame, epoch) counted.
+uint32_t *fused_frame_totals(void *frame, uint32_t epoch);
 
 }  // namespace tg
