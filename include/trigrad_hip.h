@@ -245,9 +245,9 @@ int tg_bin_frame(const tg_real *vertices, int32_t n_vertices, const int32_t *ind
                  int height, int tile_w, int tile_h, uint64_t *keys, uint32_t *values, int64_t key_capacity,
                  uint32_t *total_and_status, void *frame, size_t frame_bytes, uint32_t epoch, void *zero,
                  size_t zero_bytes, uint32_t *clear_word, void *stream);
-size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int n_tiles);
-int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int n_tiles, uint64_t *keys, uint32_t *values,
-                         uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
+size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int tiles_x, int tiles_y);
+int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int tiles_x, int tiles_y, uint64_t *keys,
+                         uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
                          size_t workspace_bytes, uint32_t *status, int *result_in_alt, void *stream);
 
 /* ---- bary matrices ---------------------------------------------------------- */

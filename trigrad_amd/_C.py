@@ -349,8 +349,9 @@ def bin_frame(vertices, indices, width, height, tile_width, tile_height, capacit
     need = int(lib.tg_bin_frame_workspace_bytes(M, capacity, width, height, tile_width, tile_height))
     frame, frame_bytes, epoch = _next_frame_state(dev, need)
     pair = frame[frame_bytes:frame_bytes + 8].view(torch.int32)
-    ws_bytes = int(lib.tg_build_frame_lists_workspace_bytes(capacity, T))
-    b = dict(capacity=capacity, epoch=epoch, frame=frame, total_and_status=pair, n_tiles=T, ws_bytes=ws_bytes,
+    tiles = (-(-width // tile_width), -(-height // tile_height))
+    ws_bytes = int(lib.tg_build_frame_lists_workspace_bytes(capacity, *tiles))
+    b = dict(capacity=capacity, epoch=epoch, frame=frame, total_and_status=pair, tiles=tiles, ws_bytes=ws_bytes,
              keys=torch.empty((capacity,), dtype=torch.int64, device=dev),
              values=torch.empty((capacity,), dtype=torch.int32, device=dev),
              keys_alt=torch.empty((capacity,), dtype=torch.int64, device=dev),
@@ -358,8 +359,8 @@ def bin_frame(vertices, indices, width, height, tile_width, tile_height, capacit
              offsets=torch.empty((T + 1,), dtype=torch.int32, device=dev),
              status=torch.empty((1,), dtype=torch.int32, device=dev),
              ws=torch.empty((max(ws_bytes, 4),), dtype=torch.uint8, device=dev))
-    # the sort's own histogram route (more than 65536 tiles) clears its workspace itself
-    zero_bytes = ws_bytes if T <= 65536 else 0
+    # the sort's own histogram route (more than 256 tile columns or rows) clears its workspace itself
+    zero_bytes = ws_bytes if max(tiles) <= 256 else 0
     with _on_device(dev):
         _lib.check(lib.tg_bin_frame(_ptr(vertices), vertices.shape[0], _ptr(indices), M, width, height, tile_width, tile_height,
                                     _ptr(b["keys"]), _ptr(b["values"]), capacity, _ptr(pair), _ptr(frame),
@@ -378,7 +379,7 @@ def build_frame_lists(binned, n_keys):
     _key_count_hint[dev.index] = n_keys
     in_alt = C.c_int(0)
     with _on_device(dev):
-        _lib.check(lib.tg_build_frame_lists(_ptr(b["frame"]), b["epoch"], n_keys, b["n_tiles"], _ptr(b["keys"]), _ptr(b["values"]),
+        _lib.check(lib.tg_build_frame_lists(_ptr(b["frame"]), b["epoch"], n_keys, *b["tiles"], _ptr(b["keys"]), _ptr(b["values"]),
                                             _ptr(b["keys_alt"]), _ptr(b["values_alt"]), _ptr(b["offsets"]), _ptr(b["ws"]),
                                             b["ws_bytes"], _ptr(b["status"]), C.byref(in_alt), _stream(b["keys"])),
                    "tg_build_frame_lists")

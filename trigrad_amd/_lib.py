@@ -50,8 +50,8 @@ SIGNATURES = {
     "tg_bin_frame_supported": (_i, [_i, _i, _i, _i]),
     "tg_bin_frame_workspace_bytes": (_sz, [_i32, _i64, _i, _i, _i, _i]),
     "tg_bin_frame": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _p, _i64, _p, _p, _sz, C.c_uint32, _p, _sz, _p, _p]),
-    "tg_build_frame_lists_workspace_bytes": (_sz, [_i64, _i]),
-    "tg_build_frame_lists": (_i, [_p, C.c_uint32, _i64, _i, _p, _p, _p, _p, _p, _p, _sz, _p, C.POINTER(_i), _p]),
+    "tg_build_frame_lists_workspace_bytes": (_sz, [_i64, _i, _i]),
+    "tg_build_frame_lists": (_i, [_p, C.c_uint32, _i64, _i, _i, _p, _p, _p, _p, _p, _p, _sz, _p, C.POINTER(_i), _p]),
     "tg_bary": (_i, [_p, _i32, _p, _i32, _p, _p]),
     "tg_list_bound_words": (_sz, [_i64, _i]),
     "tg_list_bounds": (_i, [_p, _i32, _p, _i32, _p, _p, _p, _i, _p, _p, _p, _p]),

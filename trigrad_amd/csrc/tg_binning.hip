@@ -572,63 +572,28 @@ __device__ __forceinline__ uint32_t frame_tile_prefix(uint64_t *states, int tile
     return prefix;
 }
 
-// Like count_tile_digits with short lane loops: a rectangle of up to kLaneRectShort tiles is walked by its lane,
-// larger ones by the whole wave, 64 tiles at a time.
-constexpr uint32_t kLaneRectShort = 6;
-__device__ __forceinline__ void count_tile_digits_short(const Rect &r, uint32_t count, int tiles_x, const PassPlan &plan,
-                                                        uint32_t (*hist)[kRadix]) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int shift0 = plan.shift[0] - 32, shift1 = plan.shift[1] - 32;
-    const uint32_t mask0 = (1u << plan.bits[0]) - 1, mask1 = (1u << plan.bits[1]) - 1;
-    const bool two = plan.passes > 1;
-    if (count > 0 && count <= kLaneRectShort) {
-        int tx = r.x0, ty = r.y0;
-        for (uint32_t i = 0; i < count; i++) {
-            const uint32_t tile = (uint32_t)(ty * tiles_x + tx);
-            atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
-            if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
-            if (++ty > r.y1) { ty = r.y0; tx++; }
-        }
-    }
-    uint64_t large = __builtin_amdgcn_ballot_w64(count > kLaneRectShort);
-    while (large) {
-        const int src = __builtin_ctzll(large);
-        large &= large - 1;
-        const int x0 = __shfl(r.x0, src, kWave), y0 = __shfl(r.y0, src, kWave);
-        const int ny = __shfl(r.y1, src, kWave) - y0 + 1, nx = __shfl(r.x1, src, kWave) - x0 + 1;
-        // lane l takes the tiles l, l + 64, ... of the rectangle in column-major order (column = tile x)
-        int col = lane / ny, row = lane % ny;
-        const int col_step = kWave / ny, row_step = kWave % ny;
-        while (col < nx) {
-            const uint32_t tile = (uint32_t)((y0 + row) * tiles_x + x0 + col);
-            atomicAdd(&hist[0][(tile >> shift0) & mask0], 1u);
-            if (two) atomicAdd(&hist[1][(tile >> shift1) & mask1], 1u);
-            col += col_step;
-            row += row_step;
-            if (row >= ny) { row -= ny; col++; }
-        }
-    }
-}
-
 __global__ __launch_bounds__(kScanThreads) void frame_scan_kernel(const real4 *__restrict__ vertices, int n_vertices,
                                                                   const int32_t *__restrict__ indices, int n_triangles, int W, int H,
                                                                   int tw, int th, int tiles_x, int tiles_y, uint32_t epoch,
                                                                   uint32_t *__restrict__ tri_offsets, real4 *__restrict__ records,
                                                                   uint32_t *total_and_status, uint32_t *ticket, uint64_t *states,
                                                                   int n_scan_tiles, uint32_t head_capacity, uint32_t *__restrict__ heads,
-                                                                  PassPlan plan, uint32_t *totals, uint32_t *totals_next,
+                                                                  uint32_t *totals, uint32_t *totals_next,
                                                                   real *__restrict__ edges, uint32_t *zero, size_t zero_words,
                                                                   uint32_t *clear_word) {
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_wave_total[kScanThreads / kWave];
     __shared__ uint32_t s_tile_prefix;
     __shared__ uint32_t s_count[kScanTile];
-    __shared__ uint32_t s_hist[kEmitDigitPasses][kRadix];
+    // difference arrays of the keys per tile column and per tile row: a triangle adds its rows at its first column
+    // and takes them off behind its last one, likewise for the rows; the running sums are the digit counts
+    __shared__ uint32_t s_diff[kEmitDigitPasses][kRadix + 1];
+    __shared__ uint32_t s_digit_wave[kScanThreads / kWave];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    if (totals && tid < kRadix)
-        for (int p = 0; p < kEmitDigitPasses; p++) s_hist[p][tid] = 0;
+    if (totals && tid <= kRadix)
+        for (int p = 0; p < kEmitDigitPasses; p++) s_diff[p][tid] = 0;
     if (tid == 0) {
         uint32_t mine = blockIdx.x;  // no ticket: the whole grid is resident
         if (ticket) {
@@ -674,14 +639,25 @@ __global__ __launch_bounds__(kScanThreads) void frame_scan_kernel(const real4 *_
             rect = r;
         }
         s_count[k * kScanThreads + tid] = count;
-        if (totals) count_tile_digits_short(rect, count, tiles_x, plan, s_hist);
+        if (totals && count) {
+            const uint32_t nx = (uint32_t)(rect.x1 - rect.x0 + 1), ny = (uint32_t)(rect.y1 - rect.y0 + 1);
+            atomicAdd(&s_diff[0][rect.x0], ny);
+            atomicAdd(&s_diff[0][rect.x1 + 1], 0u - ny);
+            atomicAdd(&s_diff[1][rect.y0], nx);
+            atomicAdd(&s_diff[1][rect.y1 + 1], 0u - nx);
+        }
     }
     lds_barrier();
-    if (totals && tid < kRadix)
-        for (int p = 0; p < plan.passes; p++) {
-            const uint32_t c = s_hist[p][tid];
-            if (c) atomicAdd(&totals[p * kRadix + tid], c);
-        }
+    if (totals) {  // running sums of the difference arrays: waves 0..3 take the columns, 4..7 the rows
+        static_assert(kScanThreads == kEmitDigitPasses * kRadix, "one thread per digit of the two passes");
+        const int p = tid / kRadix, d = tid & (kRadix - 1);
+        const uint32_t digit_incl = wave_inclusive_scan_u32(s_diff[p][d]);
+        if (lane == kWave - 1) s_digit_wave[wave] = digit_incl;
+        lds_barrier();
+        uint32_t keys_of_digit = digit_incl;
+        for (int w = p * (kRadix / kWave); w < wave; w++) keys_of_digit += s_digit_wave[w];
+        if (keys_of_digit) atomicAdd(&totals[p * kRadix + d], keys_of_digit);
+    }
     uint32_t x[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) x[k] = s_count[tid * 4 + k];
@@ -744,7 +720,7 @@ struct FrameKey {
     uint32_t tile_id;
 };
 __device__ __forceinline__ FrameKey frame_key(const real4 *__restrict__ records, int n_triangles, int t, uint32_t local,
-                                              const real *__restrict__ edges, int tiles_x) {
+                                              const real *__restrict__ edges, int tiles_x, int column_bits) {
     const real4 r0 = records[t], r1 = records[(int64_t)n_triangles + t], r2 = records[2 * (int64_t)n_triangles + t];
     FrameKey k;
     k.A = r0.x; k.B = r0.y; k.C = r0.z;
@@ -758,7 +734,8 @@ __device__ __forceinline__ FrameKey frame_key(const real4 *__restrict__ records,
     const int tx = int_of_real(r0.w) + (int)col, ty = int_of_real(r2.z) + row;
     k.xmin = edges[tx]; k.xmax = edges[tx + 1];  // a few hundred scalars that every key reads: they stay in cache
     k.ymin = edges[tiles_x + 1 + ty]; k.ymax = edges[tiles_x + 2 + ty];
-    k.tile_id = (uint32_t)(ty * tiles_x + tx);
+    // the key's high word: the tile number, or for the sort by column and row the pair ty << column_bits | tx
+    k.tile_id = column_bits ? ((uint32_t)ty << column_bits) | (uint32_t)tx : (uint32_t)(ty * tiles_x + tx);
     return k;
 }
 // The clip passes that may change the key's polygon (bit b: pass b of render.cu:254-257), see above.
@@ -780,7 +757,8 @@ __global__ __launch_bounds__(kEmitThreads) void frame_emit_kernel(const real4 *_
                                                                   int n_triangles, const uint32_t *__restrict__ total_and_status,
                                                                   uint32_t key_capacity, const uint32_t *__restrict__ heads,
                                                                   uint32_t head_capacity, const real *__restrict__ edges, int tiles_x,
-                                                                  uint64_t *__restrict__ keys, uint32_t *__restrict__ payload) {
+                                                                  int column_bits, uint64_t *__restrict__ keys,
+                                                                  uint32_t *__restrict__ payload) {
     __shared__ EmitLds L;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -838,7 +816,7 @@ __global__ __launch_bounds__(kEmitThreads) void frame_emit_kernel(const real4 *_
         if (at < n_keys) {
             const uint32_t m = L.owner[in_chunk];
             const int t = t_first + (m ? (int)m - 1 : 0);  // every key position has a mark at or before it
-            const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x);
+            const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x, column_bits);
             const uint32_t todo = frame_key_passes(key);
             if (todo == 0) {
                 real md = std::numeric_limits<real>::max();
@@ -878,7 +856,7 @@ __global__ __launch_bounds__(kEmitThreads) void frame_emit_kernel(const real4 *_
         uint32_t todo = e & 15u;
         const uint32_t m = L.owner[in_chunk];
         const int t = t_first + (m ? (int)m - 1 : 0);
-        const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x);
+        const FrameKey key = frame_key(records, n_triangles, t, at - tri_offsets[t], edges, tiles_x, column_bits);
         L.poly.x[0][tid] = key.ax; L.poly.y[0][tid] = key.ay;
         L.poly.x[1][tid] = key.bx; L.poly.y[1][tid] = key.by;
         L.poly.x[2][tid] = key.cx; L.poly.y[2][tid] = key.cy;
@@ -1222,17 +1200,17 @@ extern "C" int tg_bin_frame(const real *vertices, int32_t n_vertices, const int3
     static int resident_cache[kMaxDevices] = {0};
     uint32_t *ticket = f.ticket;
     if (n_scan_tiles <= resident_workgroups((const void *)frame_scan_kernel, kScanThreads, resident_cache)) ticket = nullptr;
-    const PassPlan plan = tile_pass_plan(tiles_x * tiles_y);
-    const bool count_digits = binning_counts_digits(tiles_x * tiles_y);
+    const GridPlan grid = grid_plan(tiles_x, tiles_y);
     TG_LAUNCH(frame_scan_kernel, dim3(n_scan_tiles), dim3(kScanThreads), 0, s, (const real4 *)vertices, n_vertices, indices, n_triangles,
               width, height, tile_w, tile_h, tiles_x, tiles_y, epoch, f.tri_offsets, f.records, total_and_status, ticket, f.states,
-              n_scan_tiles, f.head_capacity, f.heads, plan, count_digits ? fused_frame_totals(frame, epoch) : (uint32_t *)nullptr,
+              n_scan_tiles, f.head_capacity, f.heads, grid.on ? fused_frame_totals(frame, epoch) : (uint32_t *)nullptr,
               fused_frame_totals(frame, epoch + 1), f.edges, (uint32_t *)zero, zero_bytes / 4, clear_word);
     if (int e = check_launch("frame_scan_kernel")) return e;
     if (key_capacity == 0) return 0;
     // for every key position the buffers hold: the kernel reads K and the workgroups behind it leave at once
     TG_LAUNCH(frame_emit_kernel, dim3((unsigned)ceil_div64(key_capacity, kEmitChunk)), dim3(kEmitThreads), 0, s, f.records, f.tri_offsets,
-              n_triangles, total_and_status, (uint32_t)key_capacity, f.heads, f.head_capacity, f.edges, tiles_x, keys, values);
+              n_triangles, total_and_status, (uint32_t)key_capacity, f.heads, f.head_capacity, f.edges, tiles_x,
+              grid.on ? grid.column_bits : 0, keys, values);
     return check_launch("frame_emit_kernel");
 #endif
 }

@@ -29,6 +29,7 @@
 // (then no workgroup has to finish for another to start), by the workgroup ids,
 // which saves the serialised same-address atomics.  Waits are bounded
 // (TG_STATUS_LOOKBACK_TIMEOUT).
+#include "tg_scan.hpp"
 #include "tg_sort_plan.hpp"
 
 namespace tg {
@@ -201,12 +202,14 @@ __global__ __launch_bounds__(kSweepThreads) void sort_sweep_kernel(const uint64_
                                                                   uint64_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
                                                                   int64_t n, int shift, uint32_t mask,
                                                                   const uint32_t *__restrict__ bases, int totals_given,
-                                                                  uint32_t *lookback, uint32_t *ticket, uint32_t *status) {
+                                                                  uint32_t *lookback, uint32_t *ticket, uint32_t *status,
+                                                                  int unpad_bits, int tiles_x, uint32_t *tile_count) {
     constexpr int kDigits = 1 << BITS;
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_global_delta[kRadix];
     __shared__ uint32_t s_scan_wave[kSweepWaves];
     __shared__ uint32_t s_base_wave[kSweepWaves];
+    __shared__ uint32_t s_several_tiles[kRadix];  // with tile_count: the digit's pairs of this sort tile belong to more than one tile
     // The ranking counters are dead once every pair knows its place in the tile,
     // so they share LDS with the permutation buffer (51 KB: three workgroups per CU).
     __shared__ __align__(16) unsigned char s_raw[kSortTile * 12];
@@ -368,13 +371,45 @@ __global__ __launch_bounds__(kSweepThreads) void sort_sweep_kernel(const uint64_
     if (tid < kRadix) s_global_delta[tid] = base + prefix - local_start;
 
     __syncthreads();
+    if (tile_count) {
+        if (tid < kRadix) {
+            // the last pass of a sort by tile column and row: the pairs of a row lie together in LDS, ordered by column.
+            // Mostly they are one tile's (a sort tile spans few columns): then the row's count is that tile's.
+            uint32_t several = 0;
+            if (owns_digit && published > 0) {
+                const uint32_t hi_first = (uint32_t)(s_keys[local_start] >> 32), hi_last = (uint32_t)(s_keys[local_start + published - 1] >> 32);
+                if (hi_first == hi_last)
+                    atomicAdd(&tile_count[(hi_first >> unpad_bits) * (uint32_t)tiles_x + (hi_first & ((1u << unpad_bits) - 1))], published);
+                else
+                    several = 1;
+            }
+            s_several_tiles[tid] = several;
+        }
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < kSweepItems; i++) {
         const int pos = i * kSweepThreads + tid;
         if (pos < n_valid) {
-            const uint64_t k = s_keys[pos];
+            uint64_t k = s_keys[pos];
             const uint32_t d = (uint32_t)(k >> shift) & mask;
             const uint32_t g = s_global_delta[d] + (uint32_t)pos;
+            if (unpad_bits) {
+                // the last pass of a sort by tile column and row: the high word ty << unpad_bits | tx becomes the tile
+                // number.  Where a row's pairs here belong to several tiles, each run of one tile adds its length to
+                // the tile's count (its first and its last pair add what they know of it).
+                const uint32_t hi = (uint32_t)(k >> 32);
+                const uint32_t tile_id = (hi >> unpad_bits) * (uint32_t)tiles_x + (hi & ((1u << unpad_bits) - 1));
+                k = ((uint64_t)tile_id << 32) | (uint32_t)k;
+                if (tile_count && s_several_tiles[d]) {
+                    const uint32_t before = pos > 0 ? (uint32_t)(s_keys[pos - 1] >> 32) : ~hi;
+                    const uint32_t after = pos + 1 < n_valid ? (uint32_t)(s_keys[pos + 1] >> 32) : ~hi;
+                    const bool first = before != hi, last = after != hi;
+                    if (first && last) atomicAdd(&tile_count[tile_id], 1u);
+                    else if (first) atomicAdd(&tile_count[tile_id], 0u - (uint32_t)pos);
+                    else if (last) atomicAdd(&tile_count[tile_id], (uint32_t)pos + 1u);
+                }
+            }
             keys_out[g] = k;
             vals_out[g] = s_vals[pos];
         }
@@ -589,17 +624,50 @@ struct MediumSegLds {
     SegLds lds;
     uint32_t ex_keys[kSegMediumCap], ex_vals[kSegMediumCap];
 };
-__global__ __launch_bounds__(kSortThreads) void segment_sort_small_kernel(uint64_t *keys, uint32_t *vals,
-                                                                          const int32_t *__restrict__ offsets, int n_segments) {
+// Where the segments lie: either `offsets` holds their bounds (tile_ranges_kernel wrote them), or -- tile_count given --
+// the last sweep of a sort by tile column and row left every tile's number of pairs, and the bounds are made here:
+// a tile's first pair comes behind all pairs of the rows above it (row_totals, the digit totals of the sweep over
+// the rows) and of the tiles to its left in its row.  The kernel then writes `offsets`.
+__global__ __launch_bounds__(kSortThreads) void segment_sort_small_kernel(uint64_t *keys, uint32_t *vals, int32_t *offsets,
+                                                                          int n_segments, const uint32_t *__restrict__ tile_count,
+                                                                          const uint32_t *__restrict__ row_totals, int tiles_x,
+                                                                          uint32_t n_pairs) {
     __shared__ union SmallLds {
         WaveSegLds wave[kSortWaves];
         MediumSegLds medium;
     } s;
+    __shared__ int s_bounds[kSortWaves + 1];
     const int wave = threadIdx.x / kWave;
     const int first = blockIdx.x * kSortWaves;
     int bounds[kSortWaves + 1];
+    if (tile_count) {
+        const int lane = threadIdx.x & (kWave - 1);
+        const int t = first + wave;
+        if (t < n_segments) {
+            const int ty = t / tiles_x, tx = t - ty * tiles_x;
+            uint32_t sum = 0;
+            for (int d = lane; d < ty; d += kWave) sum += row_totals[d];
+            for (int x = lane; x < tx; x += kWave) sum += tile_count[t - tx + x];
+            sum = wave_sum(sum);
+            if (lane == 0) {
+                // counts of a sort whose wait expired (the status word says so) may be anything: stay inside the arrays
+                sum = sum < n_pairs ? sum : n_pairs;
+                const uint32_t length = tile_count[t];
+                s_bounds[wave] = (int)sum;
+                offsets[t] = (int32_t)sum;
+                const int end = (int)(length < n_pairs - sum ? sum + length : n_pairs);
+                if (wave == kSortWaves - 1 || t == n_segments - 1) s_bounds[wave + 1] = end;
+                if (t == n_segments - 1) offsets[n_segments] = end;
+            }
+        }
+        __syncthreads();
+        const int last = min(kSortWaves, n_segments - first);  // segments of this workgroup
 #pragma unroll
-    for (int w = 0; w <= kSortWaves; w++) bounds[w] = offsets[min(first + w, n_segments)];
+        for (int w = 0; w <= kSortWaves; w++) bounds[w] = s_bounds[min(w, last)];
+    } else {
+#pragma unroll
+        for (int w = 0; w <= kSortWaves; w++) bounds[w] = offsets[min(first + w, n_segments)];
+    }
     bool any_medium = false;
     int start = 0, n = 0;
 #pragma unroll
@@ -763,17 +831,19 @@ __global__ __launch_bounds__(kSortThreads) void tile_ranges_kernel(const uint64_
 template <int BITS>
 static void launch_sweep(dim3 grid, hipStream_t s, const uint64_t *kin, const uint32_t *vin, uint64_t *kout, uint32_t *vout,
                          int64_t n, int shift, uint32_t mask, const uint32_t *bases, int totals_given, uint32_t *lookback,
-                         uint32_t *ticket, uint32_t *status) {
+                         uint32_t *ticket, uint32_t *status, int unpad_bits, int tiles_x, uint32_t *tile_count) {
     hipLaunchKernelGGL(sort_sweep_kernel<BITS>, grid, dim3(kSweepThreads), 0, s, kin, vin, kout, vout, n, shift, mask, bases,
-                       totals_given, lookback, ticket, status);
+                       totals_given, lookback, ticket, status, unpad_bits, tiles_x, tile_count);
 }
 
 // The sweeps of `plan` over (keys, values) <-> (keys_alt, values_alt).  bases: per pass kRadix words, the
 // exclusive scan of the digit totals or (totals_given) the totals; lookback: per pass n_sort_tiles * kRadix
 // words, zero; tickets: one word per pass, zero.
+// unpad_bits, tiles_x, tile_count: for the last pass of a sort by tile column and row (see the kernel), else 0.
 static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, const uint32_t *bases, int totals_given,
                       uint32_t *lookback, uint32_t *tickets, uint64_t *keys, uint32_t *values, uint64_t *keys_alt,
-                      uint32_t *values_alt, int64_t n, uint32_t *status, hipStream_t s) {
+                      uint32_t *values_alt, int64_t n, uint32_t *status, hipStream_t s, int unpad_bits = 0, int tiles_x = 0,
+                      uint32_t *tile_count = nullptr) {
     uint64_t *kin = keys, *kout = keys_alt;
     uint32_t *vin = values, *vout = values_alt;
     // 534 same-address ticket atomics cost 6 us per pass; a grid that fits the device whole takes its
@@ -789,12 +859,15 @@ static int run_sweeps(const char *fn, const PassPlan &plan, int n_sort_tiles, co
         uint32_t *lb = lookback + (size_t)p * lookback_words_per_pass(n_sort_tiles);
         uint32_t *ticket = whole_grid_resident ? (uint32_t *)nullptr : tickets + p;
         const uint32_t *b = bases + (size_t)p * kRadix * (totals_given ? kTotalsStride : 1);
+        const bool last = p == plan.passes - 1;
+        const int ub = last ? unpad_bits : 0;
+        uint32_t *tc = last ? tile_count : (uint32_t *)nullptr;
         switch (plan.bits[p]) {
-        case 8: launch_sweep<8>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
-        case 7: launch_sweep<7>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
-        case 6: launch_sweep<6>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
-        case 5: launch_sweep<5>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
-        default: launch_sweep<4>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status); break;
+        case 8: launch_sweep<8>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status, ub, tiles_x, tc); break;
+        case 7: launch_sweep<7>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status, ub, tiles_x, tc); break;
+        case 6: launch_sweep<6>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status, ub, tiles_x, tc); break;
+        case 5: launch_sweep<5>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status, ub, tiles_x, tc); break;
+        default: launch_sweep<4>(grid, s, kin, vin, kout, vout, n, plan.shift[p], mask, b, totals_given, lb, ticket, status, ub, tiles_x, tc); break;
         }
         if (int e = check_launch(fn)) return e;
         uint64_t *tk = kin; kin = kout; kout = tk;
@@ -819,11 +892,16 @@ static int run_passes(const char *fn, const PassPlan &plan, const SortLayout &L,
 }
 
 // Tile ranges of keys that are ordered by tile, then every tile's segment sorted by its depth bits in place.
+// With tile_count (the last sweep counted every tile's pairs) the ranges come from the counts, inside the segment kernel.
 static int ranges_and_segments(uint64_t *k, uint32_t *v, uint64_t *k_other, uint32_t *v_other, int64_t n, int n_tiles,
-                               int32_t *offsets, hipStream_t s) {
-    TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n + 1, kSortThreads)), dim3(kSortThreads), 0, s, k, n, n_tiles, offsets);
-    if (int e = check_launch("tile_ranges_kernel")) return e;
-    TG_LAUNCH(segment_sort_small_kernel, dim3(ceil_div(n_tiles, kSortWaves)), dim3(kSortThreads), 0, s, k, v, offsets, n_tiles);
+                               int32_t *offsets, hipStream_t s, const uint32_t *tile_count = nullptr,
+                               const uint32_t *row_totals = nullptr, int tiles_x = 0) {
+    if (!tile_count) {
+        TG_LAUNCH(tile_ranges_kernel, dim3((unsigned)ceil_div64(n + 1, kSortThreads)), dim3(kSortThreads), 0, s, k, n, n_tiles, offsets);
+        if (int e = check_launch("tile_ranges_kernel")) return e;
+    }
+    TG_LAUNCH(segment_sort_small_kernel, dim3(ceil_div(n_tiles, kSortWaves)), dim3(kSortThreads), 0, s, k, v, offsets, n_tiles,
+              tile_count, row_totals, tiles_x, (uint32_t)n);
     if (int e = check_launch("segment_sort_small_kernel")) return e;
     TG_LAUNCH(segment_sort_large_kernel, dim3(n_tiles < kSegLargeGrid ? n_tiles : kSegLargeGrid), dim3(kSortThreads), 0, s, k, v,
               k_other, v_other, offsets, n_tiles);
@@ -1016,15 +1094,23 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
 }
 
 // ---- the tile lists of a frame whose keys tg_bin_frame emitted ------------------------------------------
-extern "C" size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int n_tiles) {
-    return tg_build_tile_lists_workspace_bytes(n_keys, n_tiles);
+// Workspace: the sweeps' tickets, their look-back words, then one count per tile (and one to spare).
+static size_t frame_lists_count_offset(int64_t n_keys, int n_tiles) { return kFrameSortHeadBytes + build_lookback_bytes(n_keys, n_tiles); }
+
+extern "C" size_t tg_build_frame_lists_workspace_bytes(int64_t n_keys, int tiles_x, int tiles_y) {
+    if (n_keys < 0 || n_keys > kSortMaxN || tiles_x <= 0 || tiles_y <= 0 || (int64_t)tiles_x * tiles_y > 0x7fffffff) return 0;
+    const int n_tiles = tiles_x * tiles_y;
+    if (!grid_plan(tiles_x, tiles_y).on) return tg_tile_list_sort_workspace_bytes(n_keys, n_tiles);
+    // two passes of at most 256 digits each
+    return kFrameSortHeadBytes + 2 * lookback_words_per_pass(ceil_div64(n_keys > 0 ? n_keys : 1, kSortTile)) * 4 + (size_t)(n_tiles + 1) * 4;
 }
 
-extern "C" int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int n_tiles, uint64_t *keys, uint32_t *values,
-                                    uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
+extern "C" int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys, int tiles_x, int tiles_y, uint64_t *keys,
+                                    uint32_t *values, uint64_t *keys_alt, uint32_t *values_alt, int32_t *offsets, void *workspace,
                                     size_t workspace_bytes, uint32_t *status, int *result_in_alt, void *stream) {
-    if (n_keys < 0 || n_keys > kSortMaxN || n_tiles <= 0 || !frame || !result_in_alt || !offsets) {
-        set_error("tg_build_frame_lists: n_keys must be in [0, 2^30), n_tiles positive, frame state, offsets and result_in_alt given");
+    if (n_keys < 0 || n_keys > kSortMaxN || tiles_x <= 0 || tiles_y <= 0 || (int64_t)tiles_x * tiles_y > 0x7fffffff || !frame ||
+        !result_in_alt || !offsets) {
+        set_error("tg_build_frame_lists: n_keys must be in [0, 2^30), tile counts positive, frame state, offsets and result_in_alt given");
         return TG_E_ARG;
     }
     *result_in_alt = 0;
@@ -1033,27 +1119,30 @@ extern "C" int tg_build_frame_lists(void *frame, uint32_t epoch, int64_t n_keys,
         set_error("tg_build_frame_lists: float build only");
         return TG_E_ARG;
     }
+    const int n_tiles = tiles_x * tiles_y;
     if (n_keys == 0) {
         TG_LAUNCH(tile_ranges_kernel, dim3(1), dim3(kSortThreads), 0, s, keys, n_keys, n_tiles, offsets);
         return check_launch("tile_ranges_kernel");
     }
-    if (!binning_counts_digits(n_tiles))
+    const GridPlan grid = grid_plan(tiles_x, tiles_y);
+    if (!grid.on)
         return sort_tile_lists_run("tg_build_frame_lists", keys, values, keys_alt, values_alt, n_keys, n_tiles, offsets, workspace,
                                    workspace_bytes, status, result_in_alt, s);
     if (int e = check_sort_buffers("tg_build_frame_lists", keys, values, keys_alt, values_alt, workspace)) return e;
-    const size_t need = build_lookback_bytes(n_keys, n_tiles) + kFrameSortHeadBytes;
+    const int n_sort_tiles = (int)ceil_div64(n_keys, kSortTile);
+    const size_t lookback_bytes = 2 * lookback_words_per_pass(n_sort_tiles) * 4;
+    const size_t need = kFrameSortHeadBytes + lookback_bytes + (size_t)(n_tiles + 1) * 4;
     if (workspace_bytes < need) {
         set_error("tg_build_frame_lists: workspace of %zu bytes, need %zu", workspace_bytes, need);
         return TG_E_WORKSPACE;
     }
     uint32_t *tickets = (uint32_t *)workspace;
     uint32_t *lookback = (uint32_t *)((char *)workspace + kFrameSortHeadBytes);
-    const PassPlan plan = tile_pass_plan(n_tiles);
-    if (int e = run_sweeps("tg_build_frame_lists", plan, (int)ceil_div64(n_keys, kSortTile), fused_frame_totals(frame, epoch), 1, lookback,
-                           tickets, keys, values, keys_alt, values_alt, n_keys, status, s))
+    uint32_t *tile_count = (uint32_t *)((char *)workspace + kFrameSortHeadBytes + lookback_bytes);
+    const uint32_t *totals = fused_frame_totals(frame, epoch);
+    if (int e = run_sweeps("tg_build_frame_lists", grid.plan, n_sort_tiles, totals, 1, lookback, tickets, keys, values, keys_alt,
+                           values_alt, n_keys, status, s, grid.column_bits, tiles_x, tile_count))
         return e;
-    uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
-    uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;
-    *result_in_alt = (plan.passes & 1);
-    return ranges_and_segments(k, v, k_other, v_other, n_keys, n_tiles, offsets, s);
+    // two passes: the sorted pairs are back in (keys, values)
+    return ranges_and_segments(keys, values, keys_alt, values_alt, n_keys, n_tiles, offsets, s, tile_count, totals + kRadix, tiles_x);
 }

@@ -106,4 +106,28 @@ uint32_t *frame_tickets(void *frame);
 // The digit totals that tg_bin_frame(frame, epoch) counted.
 uint32_t *fused_frame_totals(void *frame, uint32_t epoch);
 
+// The sort of a frame whose binning is tg_bin_frame.  A tile number ty * tiles_x + tx orders like the pair (ty, tx),
+// so two stable passes, by tile column and then by tile row, sort by tile.  The keys carry the pair as
+// ty << column_bits | tx in their high word until the second pass, which writes the tile number in its place.
+// The digits are then coordinates of the triangle's tile rectangle: every column of it holds as many keys as the
+// rectangle has rows, so the binning counts a pass's digits with two additions per triangle to a difference
+// array instead of one per key.  Up to 256 tile columns and rows; other frames sort on the bits of the tile
+// number with a histogram of their own.
+struct GridPlan {
+    bool on;
+    int column_bits, row_bits;
+    PassPlan plan;
+};
+inline GridPlan grid_plan(int tiles_x, int tiles_y) {
+    GridPlan g;
+    g.column_bits = tile_bits_of(tiles_x);
+    g.row_bits = tile_bits_of(tiles_y);
+    g.on = sizeof(real) == 4 && g.column_bits <= kRadixBits && g.row_bits <= kRadixBits;
+    g.plan = plan_passes(32, 32);
+    g.plan.passes = 2;
+    g.plan.shift[0] = 32; g.plan.bits[0] = g.column_bits;
+    g.plan.shift[1] = 32 + g.column_bits; g.plan.bits[1] = g.row_bits;
+    return g;
+}
+
 }  // namespace tg
