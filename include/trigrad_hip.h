@@ -61,6 +61,13 @@ typedef float tg_real;
 
 int tg_version(void);
 int tg_precision_bits(void); /* 32 or 64 */
+
+/* on != 0: every kernel that waits on other workgroups numbers its tiles by an
+ * atomic ticket, whatever the size of its grid, so that it only ever waits
+ * for workgroups that already run.  Slower (the tickets are same-address
+ * atomics), and safe when the device is shared; for a caller that has seen
+ * TG_STATUS_LOOKBACK_TIMEOUT.  Process-wide, like tg_profile_enable. */
+void tg_force_tickets(int on);
 const char *tg_last_error(void);
 
 /* Number of tiles of a W x H image (reference render.cu:105-106). */
@@ -299,6 +306,9 @@ int tg_list_bounds(const tg_real *vertices, int32_t n_vertices, const int32_t *i
  * reads them back instead of repeating the inside tests.  The buffer is
  * private to the two calls: its layout is theirs to change.
  * batch_bounds, far_start: tg_list_bounds' outputs, or NULL (used with per_pixel_sort only).
+ * list_status (may be NULL): the status word of the call that made the lists.  If it
+ * is not TG_STATUS_OK when the kernel runs, the lists are not read: image and depthmap
+ * are filled with NaN (ends, last 0), so that an invalid frame shows in the frame itself.
  * max_layers must be > 0 (the Python layer maps <= 0 to M+1, wrapper.py:35). */
 size_t tg_hit_mask_words(int64_t n_keys, int width, int height, int tile_w, int tile_h);
 int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_real *colors, const tg_real *opacities,
@@ -306,7 +316,7 @@ int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_
                       int tile_w, int tile_h, tg_real early_stopping_threshold, int per_pixel_sort, int max_layers,
                       tg_real *image, tg_real *depthmap, tg_real *final_weights, int32_t *ends, int32_t *last,
                       tg_real *last_depth, int32_t *fragments, uint64_t *hit_masks,
-                      const tg_real *batch_bounds, const int32_t *far_start, void *stream);
+                      const tg_real *batch_bounds, const int32_t *far_start, const uint32_t *list_status, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
 

@@ -50,9 +50,9 @@ def test_host_side_helpers_and_argument_rejection(bits):
     res = C.c_int(7)
     assert lib.tg_sort_pairs_u64_u32(None, None, None, None, 1 << 31, 64, None, 0, None, C.byref(res), None) == -1
     assert lib.tg_tile_ranges(None, 5, 10, None, None) == -1
-    assert lib.tg_render_forward(*([None] * 7), 64, 64, 64, 32, 0.0, 0, 1, *([None] * 11)) == -1
+    assert lib.tg_render_forward(*([None] * 7), 64, 64, 64, 32, 0.0, 0, 1, *([None] * 12)) == -1
     assert b"tile_w*tile_h" in lib.tg_last_error()
-    assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 11)) == -1
+    assert lib.tg_render_forward(*([None] * 7), 64, 64, 16, 16, 0.0, 0, 0, *([None] * 12)) == -1
     assert b"max_layers" in lib.tg_last_error()
     assert lib.tg_render_backward(*([None] * 17), 64, 64, 16, 16, 0.0, 0, 1, None, None, None, 4, 3, 1, None) == -1
     assert lib.tg_split_gradient_block(None, 5, None, None, None, None) == -1 and b"null pointer" in lib.tg_last_error()
@@ -73,6 +73,18 @@ def test_host_side_helpers_and_argument_rejection(bits):
     assert lib.tg_build_tile_lists(None, None, 5, 10, 0, None, None, 64, 64, 16, 16, None, None, None, None, None, None, 0, None, 0,
                                    C.byref(res), None) == -1
     assert lib.tg_sort_tile_lists(None, None, None, None, 10, 0, None, None, 0, None, C.byref(res), None) == -1
+    # the frame's binning without a wait for the host (float build) and the sort of its keys
+    assert lib.tg_bin_frame_supported(1920, 1080, 16, 16) == (1 if bits == 32 else 0)
+    assert lib.tg_bin_frame_supported(1 << 14, 1 << 14, 2, 2) == 0  # more than 2^21 tiles
+    assert lib.tg_bin_frame_workspace_bytes(10 ** 6, 3 * 10 ** 6, 1920, 1080, 16, 16) % 256 == 0
+    assert lib.tg_bin_frame_workspace_bytes(10 ** 6, 3 * 10 ** 6, 1920, 1080, 16, 16) > 52 * 10 ** 6  # records and offsets of the triangles
+    assert lib.tg_bin_frame_workspace_bytes(-1, 0, 64, 64, 16, 16) == 0
+    assert lib.tg_bin_frame(None, 0, None, 5, 64, 64, 16, 16, None, None, 0, None, None, 0, 1, None, 0, None, None) == -1
+    assert b"tg_bin_frame" in lib.tg_last_error()
+    assert lib.tg_build_frame_lists_workspace_bytes(10 ** 6, 120, 68) > 0 and lib.tg_build_frame_lists_workspace_bytes(1 << 30, 120, 68) == 0
+    assert lib.tg_build_frame_lists(None, 1, 10, 120, 68, None, None, None, None, None, None, 0, None, C.byref(res), None) == -1
+    lib.tg_force_tickets(1)
+    lib.tg_force_tickets(0)
     assert lib.tg_scan_noalloc_max_n() == 1 << 24
     assert lib.tg_scan_exclusive_u32_noalloc(None, None, (1 << 24) + 1, None, None, 256, 0, None, None) == -1
     with pytest.raises(RuntimeError, match="tg_bin_count failed with code -1"):

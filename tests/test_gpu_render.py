@@ -416,9 +416,14 @@ class _ReferenceShapedRenderer:
 
             @staticmethod
             def backward(ctx, grad_image, grad_depthmap):
-                gv, gc, go = _C.render_backward(grad_image, grad_depthmap, *ctx.saved_tensors, *ctx.args)
+                saved = ctx.saved_tensors
+                # which route render_backward takes: with the private state it walks what the forward pass saved,
+                # without it the forward kernel runs once more
+                Fn.resume_seen.append(getattr(saved[-1], "_tg_resume", None) is not None)
+                gv, gc, go = _C.render_backward(grad_image, grad_depthmap, *saved, *ctx.args)
                 return (gv, None, gc, go) + (None,) * 8
 
+        Fn.resume_seen = []
         return Fn
 
 
@@ -452,12 +457,14 @@ def test_native_surface_as_the_reference_wrapper_calls_it(mode, drop_private_sta
                                         W, H, 16, 16, m["per_pixel_sort"], ml)
     for label, got, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
         assert_close(f"{mode}: {label}", got.cpu().numpy(), w, 1e-4, 1e-6 + 2e-6 * float(np.abs(w).max()))
+    # the attribute on `ends` must survive save_for_backward, or every backward pass pays for a second forward kernel
+    assert Fn.resume_seen == [not drop_private_state]
 
 
 def test_expired_wait_is_reported_on_every_path(cuda):
     """A non-zero status word of the list kernels (a bounded look-back wait expired: the lists are invalid) raises in
-    the backward pass and at the start of the next frame, not only when timings are recorded.  No wait is provoked:
-    the status word is forged."""
+    the backward pass, at the start of the next frame and in verify_frames, not only when timings are recorded, and
+    switches the kernels to ticketed tile numbers.  No wait is provoked: the status word is forged."""
     import torch
     import trigrad_amd
     from trigrad_amd import _C
@@ -466,20 +473,88 @@ def test_expired_wait_is_reported_on_every_path(cuda):
     args = (d["vertices"], d["indices"], d["colors"], d["opacities"], 256, 256, 16, 16, 1 / 256)
     *results, resume = _C._forward_full(*args, True, False, 2000)
     image, depthmap, weights, sorted_ids, offsets, bary, ends = results[:7]
-    bad = _C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda))
-    gi = torch.ones_like(image)
-    with pytest.raises(RuntimeError, match="look-back wait timed out"):
-        _C.render_backward(gi, None, *args[:4], sorted_ids, offsets, bary, image, depthmap, weights, ends, *args[4:], False, 2000,
-                           resume=(resume[0], resume[1], bad, resume[3], resume[4]))
-    # the same through the public entry point: the next frame refuses to start
-    _C._pending_checks.append(_C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda)))
-    torch.cuda.synchronize()
-    with pytest.raises(RuntimeError, match="look-back wait timed out"):
-        trigrad_amd.render(*args[:6])
-    assert not _C._pending_checks or all(not c.checked for c in _C._pending_checks)
-    trigrad_amd.render(*args[:6])  # reported once; later frames run
-    # and a healthy frame's word is zero
-    resume[2].verify()
+    try:
+        bad = _C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda), frame=7)
+        gi = torch.ones_like(image)
+        with pytest.raises(RuntimeError, match="look-back wait timed out.*frame 7"):
+            _C.render_backward(gi, None, *args[:4], sorted_ids, offsets, bary, image, depthmap, weights, ends, *args[4:], False, 2000,
+                               resume=(resume[0], resume[1], bad, resume[3], resume[4]))
+        assert _C._tickets_forced
+        # the same through the public entry point: the next frame refuses to start
+        _C._pending_checks.append(_C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda)))
+        torch.cuda.synchronize()
+        with pytest.raises(RuntimeError, match="look-back wait timed out"):
+            trigrad_amd.render(*args[:6])
+        assert not _C._pending_checks or all(not c.checked for c in _C._pending_checks)
+        trigrad_amd.render(*args[:6])  # reported once; later frames run (their tiles numbered by ticket)
+        # a caller that only renders forward asks before it trusts its frames
+        _C._pending_checks.append(_C.StatusCheck(torch.ones((1,), dtype=torch.int32, device=cuda)))
+        with pytest.raises(RuntimeError, match="look-back wait timed out"):
+            trigrad_amd.verify_frames()
+        trigrad_amd.verify_frames()
+        # and a healthy frame's word is zero
+        resume[2].verify()
+    finally:
+        _C.force_tickets(False)
+
+
+def test_invalid_lists_show_in_the_frame(cuda):
+    """The forward kernels look at the status word of the list kernels: with a word that reports an expired wait they
+    read no list and fill image and depth map with NaN, in both compositing orders.  The word is forged."""
+    import ctypes as C
+    import torch
+    from trigrad_amd import _C, _lib
+    import scenes as S
+    d = to_device(S.config(0), cuda)
+    W = H = 256
+    v, idx, col, op = d["vertices"], d["indices"], d["colors"], d["opacities"]
+    *results, resume = _C._forward_full(v, idx, col, op, W, H, 16, 16, 1 / 256, True, False, 2000)
+    want_image, _, _, sorted_ids, offsets, bary = results[:6]
+    lib = _lib.load(32)
+    for word, pps in ((0, False), (1, False), (1, True)):
+        status = torch.full((1,), word, dtype=torch.int32, device=cuda)
+        image = torch.zeros((H, W, 4), device=cuda)
+        planes = [torch.zeros((H, W), device=cuda) for _ in range(3)]
+        ends = torch.zeros((H, W), dtype=torch.int32, device=cuda)
+        last = torch.zeros((H, W), dtype=torch.int32, device=cuda)
+        p = lambda t: C.c_void_p(t.data_ptr())
+        _lib.check(lib.tg_render_forward(p(v), p(idx), p(col), p(op), p(sorted_ids), p(offsets), p(bary), W, H, 16, 16, 1 / 256, int(pps),
+                                         2000, p(image), p(planes[0]), p(planes[1]), p(ends), p(last), p(planes[2]) if pps else None,
+                                         None, None, None, None, p(status), C.c_void_p(torch.cuda.current_stream().cuda_stream)),
+                   "tg_render_forward")
+        if word == 0:
+            assert torch.equal(image, want_image)
+        else:
+            assert torch.isnan(image).all() and torch.isnan(planes[0]).all() and int(ends.abs().max()) == 0
+
+
+def test_ticketed_tile_numbers_change_nothing(cuda, oracle):
+    """force_tickets: the kernels that wait on other workgroups take their tile numbers from an atomic ticket whatever
+    the size of the grid.  Lists and image are, bit for bit, what they are without."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import _C
+    import scenes as S
+    scene = S.config(1)
+    d = to_device(scene, cuda)
+    W, H = scene["width"], scene["height"]
+
+    def frame():
+        image, _ = trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, 16, 16, 1 / 256, False, False, -1)
+        b = _C.bin_frame(d["vertices"], d["indices"], W, H, 16, 16)
+        K = int(b["total_and_status"][0].item())
+        keys, ids, status, offsets = _C.build_frame_lists(b, K)
+        assert int(status.item()) == 0
+        return image, keys.clone(), ids.clone(), offsets.clone()
+
+    plain = frame()
+    try:
+        _C.force_tickets(True)
+        ticketed = frame()
+    finally:
+        _C.force_tickets(False)
+    for a, b in zip(plain, ticketed):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("mode", ["A_default", "B_unlimited"])

@@ -306,3 +306,24 @@ def test_frame_route_with_more_than_65536_tiles(cuda, oracle):
     np.testing.assert_array_equal(u64(fkeys), want_keys)
     np.testing.assert_array_equal(fids.cpu().numpy(), want_vals)
     np.testing.assert_array_equal(foffsets.cpu().numpy(), oracle.tile_ranges(want_keys, T))
+
+
+def test_one_frame_state_serves_two_sorting_calls(cuda):
+    """tg_build_tile_lists twice on the state of one tg_bin_setup, with more sort tiles than fit the device at once
+    (ticketed tile numbers): the second call finds its tickets at zero again and gives the same lists."""
+    import torch
+    from trigrad_amd import _C
+    import scenes as S
+    scene = S.config(3, with_target=False)
+    W, H = scene["width"], scene["height"]
+    d = to_device(scene, cuda)
+    setup = _C.bin_setup(d["vertices"], d["indices"], W, H, 16, 16)
+    K = int(setup["total_and_status"][0].item())
+    assert K > 3_200_000
+    first = [t.clone() for t in _C.build_tile_lists(setup, K)]
+    second = _C.build_tile_lists(setup, K)
+    assert int(first[2].item()) == 0 and int(second[2].item()) == 0
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    skeys = u64(first[0])
+    assert (np.diff(skeys.astype(np.uint64).view(np.int64)) >= 0).all()

@@ -468,15 +468,32 @@ class _StageTimer:
         return {name: evs[k].elapsed_time(evs[k + 1]) / 1000.0 for k, (name, _) in enumerate(self.marks)}
 
 
+_frame_counter = 0  # frames rendered by this process, for the messages of StatusCheck
+
+
+def force_tickets(on=True):
+    """Makes every kernel that waits on other workgroups number its tiles by an atomic ticket (tg_force_tickets):
+    slower, and safe when other work shares the device.  Switched on by the first wait that expires."""
+    for bits, lib in list(_lib._libs.items()) or [(32, _lib.load(32))]:
+        lib.tg_force_tickets(1 if on else 0)
+    global _tickets_forced
+    _tickets_forced = bool(on)
+
+
+_tickets_forced = False
+
+
 class StatusCheck:
     """The status word of the kernels that wait on other workgroups (TG_STATUS_*), on its way to the host.
 
     The word is copied to pinned host memory behind the kernels that write it, without a wait; `verify`
     waits for that copy (long done when the backward pass or the next frame asks) and raises RuntimeError
-    if a bounded wait expired, because the lists and everything rendered from them are then invalid."""
+    if a bounded wait expired, because the lists and everything rendered from them are then invalid (the
+    forward kernels have filled such a frame's image with NaN).  From then on the kernels take tickets."""
 
-    def __init__(self, status, what="tg_build_tile_lists"):
+    def __init__(self, status, what="tg_build_frame_lists", frame=None):
         self.what = what
+        self.frame = frame
         self.checked = False
         if status.device.type == "cuda":
             self.host = torch.empty((status.numel(),), dtype=torch.int32, pin_memory=True)
@@ -490,33 +507,54 @@ class StatusCheck:
     def ready(self):
         return self.event is None or self.event.query()
 
-    def verify(self):
-        if self.checked:
-            return
+    def failed(self):
+        """Waits for the word; True if a wait expired."""
         if self.event is not None:
             self.event.synchronize()
         self.checked = True
-        if int(self.host.max()) != 0:
-            raise RuntimeError(f"{self.what}: look-back wait timed out (status {self.host.tolist()}); the frame is invalid")
+        return int(self.host.max()) != 0
+
+    def verify(self):
+        if self.checked:
+            return
+        if self.failed():
+            force_tickets(True)
+            which = "" if self.frame is None else f" of frame {self.frame}"
+            raise RuntimeError(f"{self.what}: look-back wait timed out (status {self.host.tolist()}); the lists{which} are "
+                               "invalid and its image is NaN.  Later frames number their tiles by ticket.")
 
 
 _pending_checks = []  # status words of earlier frames that nobody has looked at yet
+_pending_lock = threading.Lock()
 
 
-def verify_finished_frames():
-    """Raises for any earlier frame whose status word has arrived and reports a timeout; never waits."""
+def verify_frames(wait=True):
+    """Raises RuntimeError if the lists of a frame rendered earlier are invalid because a bounded wait between
+    workgroups expired (its image is then NaN).  wait=True also waits for the status words still on their way, so
+    after it returns every frame rendered so far on this process is known to be good: what a caller who only
+    renders forward (no backward pass, whose first step is this check) calls before it trusts a frame.
+    wait=False looks only at the words that have arrived."""
+    with _pending_lock:
+        checks = list(_pending_checks)
+        del _pending_checks[:]
     still = []
     try:
-        while _pending_checks:
-            check = _pending_checks.pop(0)
+        while checks:
+            check = checks.pop(0)
             if check.checked:
                 continue
-            if check.ready():
+            if wait or check.ready():
                 check.verify()
             else:
                 still.append(check)
     finally:
-        _pending_checks[:0] = still
+        with _pending_lock:
+            _pending_checks[:0] = still + [c for c in checks if not c.checked]
+
+
+def verify_finished_frames():
+    """verify_frames(wait=False): never waits."""
+    verify_frames(wait=False)
 
 
 def _forward_full(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
@@ -563,10 +601,15 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
                 arrived.synchronize()
                 K, st = host.tolist()
                 if st == _as_int32(binned["epoch"]):
-                    raise RuntimeError("tg_bin_frame: wait for another workgroup timed out")
+                    # a workgroup gave up waiting for another (other work on the device): once more, with tickets
+                    if _tickets_forced:
+                        raise RuntimeError("tg_bin_frame: wait for another workgroup timed out")
+                    force_tickets(True)
+                    K = binned["capacity"] + 1
                 if K <= binned["capacity"]:
                     break
-                binned = bin_frame(vertices, indices, width, height, tile_width, tile_height, capacity=K + K // 8)
+                binned = bin_frame(vertices, indices, width, height, tile_width, tile_height,
+                                   capacity=None if st == _as_int32(binned["epoch"]) else K + K // 8)
             timer.start("sorting")
             keys, sorted_ids, sort_status, offsets = build_frame_lists(binned, K)
         else:
@@ -580,8 +623,11 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
                 keys, sorted_ids, sort_status, offsets = sort_tile_lists(keys, payload, T)
             else:  # the double build's depth keys take 64 bits and are sorted in two rounds
                 keys, sorted_ids, sort_status, offsets = sort_lists(keys, payload, K, T)
-        status_check = StatusCheck(sort_status)
-        _pending_checks.append(status_check)
+        global _frame_counter
+        _frame_counter += 1
+        status_check = StatusCheck(sort_status, frame=_frame_counter)
+        with _pending_lock:
+            _pending_checks.append(status_check)
 
         timer.start("bary_transforms")
         if bary_transforms is None:
@@ -605,10 +651,16 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
             _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
             width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
             _ptr(image), _ptr(depthmap), _ptr(final_weights), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
-            _ptr(hit_masks), _ptr(batch_bounds), _ptr(far_start), _stream(vertices)), "tg_render_forward", bits)
+            _ptr(hit_masks), _ptr(batch_bounds), _ptr(far_start), _ptr(sort_status), _stream(vertices)), "tg_render_forward", bits)
         timings = timer.stop()
-        if not disable_timing:
-            status_check.verify()  # the timer has waited for the stream anyway
+        if not disable_timing:  # the timer has waited for the stream anyway
+            if status_check.failed() and not _tickets_forced:
+                # the lists are invalid (and the image NaN): the whole frame once more, its tiles numbered by ticket
+                force_tickets(True)
+                return _forward_full(vertices, indices, colors, opacities, width, height, tile_width, tile_height,
+                                     early_stopping_threshold, disable_timing, per_pixel_sort, max_layers)
+            status_check.checked = False
+            status_check.verify()
     return (image, depthmap, final_weights, sorted_ids, offsets, bary_transforms, ends, timings,
             (last, last_depth, status_check, fragments, hit_masks))
 
@@ -649,7 +701,7 @@ def _resume_by_forward(vertices, indices, colors, opacities, sorted_ids, offsets
         _ptr(vertices), _ptr(indices), _ptr(colors), _ptr(opacities), _ptr(sorted_ids), _ptr(offsets), _ptr(bary_transforms),
         width, height, tile_width, tile_height, float(early_stopping_threshold), int(bool(per_pixel_sort)), int(max_layers),
         _ptr(image), _ptr(plane[0]), _ptr(plane[1]), _ptr(ends), _ptr(last), _ptr(last_depth), _ptr(fragments),
-        _ptr(hit_masks), None, None, _stream(vertices)), "tg_render_forward", bits)
+        _ptr(hit_masks), None, None, None, _stream(vertices)), "tg_render_forward", bits)
     return last, last_depth, None, fragments, hit_masks
 
 

@@ -29,6 +29,7 @@ SIGNATURES = {
     "tg_precision_bits": (_i, []),
     "tg_last_error": (C.c_char_p, []),
     "tg_num_tiles": (_i, [_i, _i, _i, _i]),
+    "tg_force_tickets": (None, [_i]),
     "tg_profile_enable": (None, [_i]),
     "tg_profile_report": (_i, [C.c_char_p, _sz]),
     "tg_bin_count": (_i, [_p, _i32, _p, _i32, _i, _i, _i, _i, _p, _p]),
@@ -56,7 +57,7 @@ SIGNATURES = {
     "tg_list_bound_words": (_sz, [_i64, _i]),
     "tg_list_bounds": (_i, [_p, _i32, _p, _i32, _p, _p, _p, _i, _p, _p, _p, _p]),
     "tg_hit_mask_words": (_sz, [_i64, _i, _i, _i, _i]),
-    "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "tg_render_forward": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
     "tg_render_backward": (_i, [_p] * 17 + [_i, _i, _i, _i, _f, _i, _i, _p, _p, _p, _i, _i, _i, _p]),
     "tg_split_gradient_block": (_i, [_p, _i64, _p, _p, _p, _p]),
     "tg_barycentric": (None, [_p] * 5),

@@ -58,7 +58,10 @@ ProfileScope::~ProfileScope() {
     if (slot < (int)g_profile_records.size()) (void)hipEventRecord(g_profile_records[slot].stop, stream);
 }
 
+static bool g_force_tickets = false;
+
 int resident_workgroups(const void *kernel, int threads, int *cache, size_t dynamic_lds) {
+    if (g_force_tickets) return 0;  // "unknown": the callers then number their tiles by ticket
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
     if (cache[dev] == 0) {
@@ -108,6 +111,8 @@ extern "C" int tg_num_tiles(int width, int height, int tile_w, int tile_h) {
 }
 
 extern "C" void tg_profile_enable(int on) { tg::g_profile_on = on != 0; }
+
+extern "C" void tg_force_tickets(int on) { tg::g_force_tickets = on != 0; }
 
 extern "C" int tg_profile_report(char *buffer, size_t capacity) {
     using namespace tg;

@@ -232,7 +232,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_kernel(const real4 *__re
 // totals of the tile passes, the NDC edges of the tile columns and rows, the scan's state words.  bin_init_kernel clears it and fills in the edges.
 constexpr int kRecordReals = TG_RECORD_SCALARS;  // three planes of M x 4: A B C x0 | ax ay bx by | cx cy y0 ny
 static_assert(kRecordReals == 12, "three real4 per triangle");
-constexpr int kStateTicketWords = 64;   // word 0: scan ticket; 8..15: sweep tickets
+constexpr int kStateTicketWords = 64;   // word 0: scan ticket; kSweepTicketWord..+7: sweep tickets
 constexpr int kStateTotalsWords = kEmitDigitPasses * kRadix * kTotalsStride;
 
 struct FrameState {
@@ -400,12 +400,14 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
                                                                        int tiles_x, int tiles_y, uint64_t *__restrict__ keys,
                                                                        uint32_t *__restrict__ payload, uint32_t *zero,
                                                                        size_t zero_words, uint32_t *clear_word,
-                                                                       int chunks_per_group) {
+                                                                       uint32_t *sweep_tickets, int chunks_per_group) {
     __shared__ PolyLds lds;
     __shared__ uint32_t s_offsets[kOwnerWindow];
     const int tid = threadIdx.x;
     for (size_t i = (size_t)blockIdx.x * kBinThreads + tid; i < zero_words; i += (size_t)gridDim.x * kBinThreads) zero[i] = 0;
     if (clear_word && blockIdx.x == 0 && tid == 0) *clear_word = 0;
+    // the sweeps that follow count their tickets up from zero: a frame state may serve more than one sorting call
+    if (sweep_tickets && blockIdx.x == 0 && tid < kMaxPasses) sweep_tickets[tid] = 0;
     const int64_t n_chunks = (n_keys + kBinThreads - 1) / kBinThreads;
     const int64_t chunk_end = ((int64_t)blockIdx.x + 1) * chunks_per_group < n_chunks ? ((int64_t)blockIdx.x + 1) * chunks_per_group : n_chunks;
     for (int64_t chunk = (int64_t)blockIdx.x * chunks_per_group; chunk < chunk_end; chunk++) {
@@ -1228,7 +1230,8 @@ int launch_emit_records(const char *fn, const real *records, const uint32_t *tri
     const int chunks_per_group = 1;  // more (fewer, longer-lived workgroups) measured slower: 52 against 47 us on 2.2 M keys
     const unsigned grid = (unsigned)ceil_div64(n_chunks, chunks_per_group);
     TG_LAUNCH(bin_emit_records_kernel, dim3(grid), dim3(kBinThreads), 0, s, (const real4 *)records, tri_offsets, n_triangles, n_keys,
-              owner_heads, owner_capacity, f.edges, tiles_x, tiles_y, keys, payload, zero, zero_words, clear_word, chunks_per_group);
+              owner_heads, owner_capacity, f.edges, tiles_x, tiles_y, keys, payload, zero, zero_words, clear_word,
+              zero ? f.tickets + kSweepTicketWord : (uint32_t *)nullptr, chunks_per_group);
     return check_launch(fn);
 }
 uint32_t *frame_totals(void *frame, int32_t n_triangles, int tiles_x, int tiles_y) { return frame_state(frame, n_triangles, tiles_x, tiles_y).tickets + kStateTicketWords; }

@@ -25,7 +25,22 @@ struct ForwardOut {
     real *last_depth;
     int32_t *fragments;  // (max_layers, H, W): list positions, relative to the tile's start, in blend order; may be null
     uint64_t *hit_masks; // tile order: which list entries cover which pixel, 64 entries per word (see hit_mask_chunk); may be null
+    const uint32_t *list_status;  // status word of the kernels that made the lists (TG_STATUS_*); may be null
 };
+
+// Lists whose sort gave up a wait are not to be read (unwritten entries may name anything): the frame's pixels
+// are marked instead, so that the caller sees it in the image itself.
+__device__ __forceinline__ bool lists_invalid(const ForwardOut &o) { return o.list_status && *o.list_status != TG_STATUS_OK; }
+__device__ __forceinline__ void mark_pixel_invalid(const ForwardOut &o, const PixelCoord &p) {
+    if (!p.valid) return;
+    const real nan = std::numeric_limits<real>::quiet_NaN();
+    o.image[p.index] = make_real4(nan, nan, nan, nan);
+    o.depthmap[p.index] = nan;
+    o.weights[p.index] = 0.0f;
+    o.ends[p.index] = 0;
+    if (o.last) o.last[p.index] = 0;
+    if (o.last_depth) o.last_depth[p.index] = nan;
+}
 
 __device__ __forceinline__ void write_pixel(const ForwardOut &o, const PixelCoord &p, PixelState s, int last, real last_depth) {
     // render.cu:609-618
@@ -53,8 +68,12 @@ __global__ __launch_bounds__(kTileThreads) void forward_tile_order_kernel(Raster
     const int n_waves = blockDim.x / kWave;
     const TileId tile_id = tile_of_workgroup<kTileBandForward>();
     const int tile = tile_id.index;
-    const int start = a.offsets[tile], end = a.offsets[tile + 1];
     const PixelCoord p = pixel_of_thread(a, tile_id);
+    if (lists_invalid(out)) {  // the same for the whole launch
+        mark_pixel_invalid(out, p);
+        return;
+    }
+    const int start = a.offsets[tile], end = a.offsets[tile + 1];
     publish_wave_rect(p, s_rects);
     uint64_t *const masks = out.hit_masks ? out.hit_masks + hit_mask_head_words() : nullptr;
 
@@ -291,6 +310,10 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_kernel(Raste
     __shared__ uint8_t s_touch[kStage];
     __shared__ WaveRect s_rects[kMaxTileWaves];
     const TileId tile = tile_of_workgroup<kTileBandForward>();
+    if (lists_invalid(out)) {  // the same for the whole launch
+        mark_pixel_invalid(out, pixel_of_thread(a, tile));
+        return;
+    }
     if (sizeof(Pos) < sizeof(int) && a.offsets[tile.index + 1] - a.offsets[tile.index] > kShortList) return;
     pixel_order_tile<kStage, Pos>(a, out, tile.x, tile.y, gridDim.x, s_dyn, s_touch, s_rects);
 }
@@ -304,6 +327,7 @@ __global__ __launch_bounds__(kTileThreads) void forward_pixel_order_long_lists_k
     __shared__ uint8_t s_touch[kSelectBatch];
     __shared__ WaveRect s_rects[kMaxTileWaves];
     __shared__ uint64_t s_votes[kMaxTileWaves];
+    if (lists_invalid(out)) return;  // the launch before this one has marked every pixel
     const int tiles = tiles_x * tiles_y;
     const int share = (tiles + (int)gridDim.x - 1) / (int)gridDim.x;
     const int first = blockIdx.x * share, past = min(first + share, tiles);
@@ -393,7 +417,7 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
                                  int tile_w, int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers,
                                  real *image, real *depthmap, real *final_weights, int32_t *ends, int32_t *last,
                                  real *last_depth, int32_t *fragments, uint64_t *hit_masks, const real *batch_bounds,
-                                 const int32_t *far_start, void *stream) {
+                                 const int32_t *far_start, const uint32_t *list_status, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
         set_error("tg_render_forward: null pointer");
@@ -414,7 +438,8 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
         set_error("tg_render_forward: fragments are saved only with per_pixel_sort and max_layers <= %d", TG_MAX_SAVED_LAYERS);
         return TG_E_ARG;
     }
-    ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments, per_pixel_sort ? nullptr : hit_masks};
+    ForwardOut o{(real4 *)image, depthmap, final_weights, ends, last, last_depth, fragments, per_pixel_sort ? nullptr : hit_masks,
+                 list_status};
     const TileLaunch tl = tile_launch(width, height, tile_w, tile_h, per_pixel_sort ? pixel_order_threads(kTileThreads) : kTileThreads);
     const dim3 grid = tl.grid;
     const int n_threads = tl.threads;

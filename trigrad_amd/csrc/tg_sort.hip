@@ -1085,7 +1085,7 @@ extern "C" int tg_build_tile_lists(const real *records, const uint32_t *tri_offs
     const int tiles_x = ceil_div(width, tile_w), tiles_y = ceil_div(height, tile_h);
     uint32_t *tickets = frame_tickets(frame);
     if (int e = run_sweeps("tg_build_tile_lists", plan, (int)ceil_div64(n_keys, kSortTile), frame_totals(frame, n_triangles, tiles_x, tiles_y),
-                           1, lookback, tickets + 8, keys, values, keys_alt, values_alt, n_keys, status, s))
+                           1, lookback, tickets + kSweepTicketWord, keys, values, keys_alt, values_alt, n_keys, status, s))
         return e;
     uint64_t *k = (plan.passes & 1) ? keys_alt : keys, *k_other = (plan.passes & 1) ? keys : keys_alt;
     uint32_t *v = (plan.passes & 1) ? values_alt : values, *v_other = (plan.passes & 1) ? values : values_alt;

@@ -78,6 +78,7 @@ inline SortLayout sort_layout(int64_t n, int passes) {
     L.total = o;
     return L;
 }
+constexpr int kSweepTicketWord = 8;  // the sweeps' tickets inside the frame state of tg_bin_setup
 constexpr int kTotalsStride = 1;  // words between two digit totals (a cache line each was tried: the atomics got no faster)
 
 
