@@ -31,10 +31,62 @@ sys.path.insert(1, os.path.join(ROOT, "tests"))  # the seeded scene generators l
 
 HBM_PEAK_GBS = 8000.0
 
-# Bytes per launch of sort_sweep_kernel that pass the L2 on their way to the fabric, measured with rocprofv3 --pmc: read and
-# write requests by size (and, agreeing within 0.2 %, FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB plain copy), keyed by
-# the number of pairs it was measured on (profiles/config2_hbm_traffic_counters.md).
-MEASURED_SWEEP_TRAFFIC = {2186877: 57.0e6}
+# Bytes per launch of sort_sweep_kernel that pass the L2 on their way to the fabric are measured with rocprofv3 --pmc (read
+# and write requests by size, and FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB plain copy) and written into this summary as a
+# line "sort_sweep_kernel traffic_bytes_per_launch=<bytes> keys=<K> commit=<hash>"; the bench line quotes it only for that K.
+TRAFFIC_SUMMARY = os.path.join("profiles", "config2_hbm_traffic_counters.md")
+
+
+def measured_sweep_traffic(n_keys):
+    """-> (bytes per launch or None, where the figure comes from)"""
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_SUMMARY)).read()
+    except OSError:
+        return None, None
+    for line in text.splitlines():
+        if line.startswith("sort_sweep_kernel traffic_bytes_per_launch="):
+            fields = dict(f.split("=", 1) for f in line.split()[1:])
+            if int(fields.get("keys", -1)) == n_keys:
+                return float(fields["traffic_bytes_per_launch"]), f"{TRAFFIC_SUMMARY} @ {fields.get('commit', '?')}"
+    return None, f"{TRAFFIC_SUMMARY} holds no measurement for K={n_keys}"
+
+
+def cpu_oracle_baseline(scene, mode, W, H, cores):
+    """The CPU oracle (a restatement of the reference's algorithm; the reference has no CPU render path) on the same frame:
+    per-stage wall time, once on one thread and, after a warm-up, as the median of three runs with OpenMP on `cores`
+    threads (binning and sort are serial code either way; the blend passes run over tiles in parallel)."""
+    import numpy as np
+    from oracle import oracle as O
+    v, i, c, o = scene["vertices"], scene["indices"], scene["colors"], scene["opacities"]
+    T = O.n_tiles(W, H, 16, 16)
+
+    def one_frame():
+        t = [time.perf_counter()]
+        em = O.bin_emit(v, i, W, H, 16, 16); t.append(time.perf_counter())
+        keys, ids = O.sort_pairs_u64(em["keys64"], em["tri"]); t.append(time.perf_counter())
+        offsets = O.tile_ranges(keys, T); t.append(time.perf_counter())
+        bm = O.bary(v, i); t.append(time.perf_counter())
+        fwd = O.forward(v, i, c, o, ids, offsets, bm, W, H, 16, 16, 1 / 256, mode["per_pixel_sort"], mode["max_layers"])
+        t.append(time.perf_counter())
+        gi = (2.0 * (fwd["image"] - scene["target"]) / fwd["image"].size).astype(np.float32)
+        O.backward(gi, np.zeros((H, W), np.float32), v, i, c, o, ids, offsets, bm, fwd, W, H, 16, 16, mode["per_pixel_sort"],
+                   mode["max_layers"])
+        t.append(time.perf_counter())
+        return dict(zip(("binning", "sort", "ranges", "bary", "forward", "backward"), np.diff(t)))
+
+    def totals(stages):
+        stages = {k: round(float(s), 4) for k, s in stages.items()}
+        fwd = sum(stages[k] for k in ("binning", "sort", "ranges", "bary", "forward"))
+        return dict(stage_seconds=stages, forward_seconds=round(fwd, 4), forward_backward_seconds=round(fwd + stages["backward"], 4))
+
+    O.set_threads(1)
+    single = totals(one_frame())
+    O.set_threads(cores)
+    one_frame()  # warm-up
+    runs = [one_frame() for _ in range(3)]
+    many = totals({k: float(np.median([r[k] for r in runs])) for k in runs[0]})
+    return single, many
+
 
 MODES = {
     "A": dict(per_pixel_sort=True, max_layers=32),    # API defaults
@@ -117,20 +169,30 @@ def main():
     _C.profile_enable(False)
     counts = _C.bin_count(d["vertices"], d["indices"], W, H, 16, 16)
     K = int(counts.sum().item())
-    passes = (_C.key_bits(T) + 7) // 8
+    # the 8-bit LSD pipeline that the byte model prices: passes over all key bits.  The frame's sort moves the pairs
+    # through memory for the tile bits only (one pass by tile column, one by tile row) and sorts the depth bits per tile
+    # in LDS (one more read and write of every pair).
+    model_passes = (_C.key_bits(T) + 7) // 8
     sweep_n, sweep_ms = prof["sort_sweep_kernel"]
     sweep_avg_s = sweep_ms / sweep_n / 1000.0
     sweep_bytes = 24.0 * K
     achieved = sweep_bytes / sweep_avg_s / 1e9
+    passes_through_memory = sweep_n // prof_steps
     per_step = {k: v[1] / prof_steps for k, v in prof.items()}
     # binning + sort + ranges: every kernel from the triangles to the sorted tile lists and their offsets
-    sort_kernels = ["fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel",
+    sort_kernels = ["fill_zero_kernel", "sort_histogram_kernel", "sort_bases_kernel", "sort_sweep_kernel", "tile_ranges_kernel",
                     "segment_sort_small_kernel", "segment_sort_large_kernel"]
     bin_sort_kernels = ["bin_count_kernel", "scan_init_kernel", "scan_lookback_kernel", "bin_emit_kernel", "bin_init_kernel",
-                        "bin_setup_kernel", "bin_emit_records_kernel", "frame_scan_kernel", "frame_emit_kernel", "tile_ranges_kernel"] + sort_kernels
+                        "bin_setup_kernel", "bin_emit_records_kernel", "frame_scan_kernel", "frame_emit_kernel"] + sort_kernels
     bin_sort_ms = sum(per_step.get(k, 0.0) for k in bin_sort_kernels)
-    bin_sort_bytes = 136.0 * M + 28.0 * K + 24.0 * passes * K + 4.0 * (T + 1)
+    # the byte model of an 8-bit LSD key pipeline: count 64 M, scan 8 M, emit 64 M + 12 K, histogram 8 K, passes 24 K each,
+    # ranges 8 K + 4 (T + 1)
+    bin_sort_bytes = 136.0 * M + 28.0 * K + 24.0 * model_passes * K + 4.0 * (T + 1)
+    # what this build's kernels move: scan (60 M read, 4 M offsets + 48 M records written), emission (records and
+    # offsets read, 12 K written), the passes through memory, the per-tile depth sort (24 K), counts and offsets per tile
+    moved_bytes = (60.0 + 52.0) * M + (52.0 * M + 12.0 * K) + 24.0 * passes_through_memory * K + 24.0 * K + 12.0 * (T + 1)
     sort_ms = sum(per_step.get(k, 0.0) for k in sort_kernels)
+    traffic, traffic_source = measured_sweep_traffic(K)
 
     out = {
         "metric": "fwd+bwd frames/s (1M tris, 1920x1080)" if args.config == 2 else f"fwd+bwd frames/s (config {args.config})",
@@ -149,16 +211,22 @@ def main():
                                f"per_pixel_sort={MODES[args.mode]['per_pixel_sort']}, max_layers={MODES[args.mode]['max_layers']}",
                    "mode": args.mode},
         "roofline": {"bound": "hbm", "kernel": "sort_sweep_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_SWEEP_TRAFFIC.get(K),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
                      "bytes_per_launch": sweep_bytes, "avg_launch_us": sweep_avg_s * 1e6},
     }
 
     extra = {
         "kernel_ms_per_step": {k: round(v, 4) for k, v in sorted(per_step.items())},
         "binning_sort_ranges": {"ms": bin_sort_ms, "algorithmic_bytes": bin_sort_bytes,
+                                "algorithmic_bytes_model": f"8-bit LSD key pipeline with {model_passes} passes over all key bits",
                                 "GBps": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9,
-                                "frac_of_hbm_peak": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS},
-        "sort_in_frame": {"keys": K, "passes": passes, "ms": sort_ms, "Gkeys_per_s": K / (sort_ms / 1000.0) / 1e9},
+                                "frac_of_hbm_peak": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
+                                "moved_bytes": moved_bytes,
+                                "moved_bytes_model": "what the kernels read and write by their access pattern (not counters)",
+                                "frac_of_hbm_peak_moved": moved_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS},
+        "sort_in_frame": {"keys": K, "passes_through_memory": passes_through_memory, "passes_of_the_byte_model": model_passes,
+                          "depth_bits": "sorted per tile in LDS: one more read and write of every pair",
+                          "ms": sort_ms, "Gkeys_per_s": K / (sort_ms / 1000.0) / 1e9},
     }
     # the blend kernels against the HBM roofline, to show that it does not bound them: compulsory bytes are
     # 148 B per list entry plus the per-pixel and per-vertex arrays (forward 28 B/pixel; backward 48 B/pixel + 64 B/vertex)
@@ -198,7 +266,7 @@ def main():
             vbuf.copy_(vals0)
         t_sort = timed(sort_once, 10, 2) - timed(copy_only, 10, 2)
         extra["sort_standalone"] = {"keys": n, "ms": t_sort, "Gkeys_per_s": n / (t_sort / 1000.0) / 1e9,
-                                    "GBps": (8.0 + 24.0 * passes) * n / (t_sort / 1000.0) / 1e9}
+                                    "GBps": (8.0 + 24.0 * model_passes) * n / (t_sort / 1000.0) / 1e9}
         # the same pairs through the sort the frame uses (tile bits through memory, depth bits per tile in LDS)
         def tile_sort_once():
             kbuf.copy_(keys0)
@@ -235,18 +303,12 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import oracle as O
         cores = min(O.max_threads(), len(os.sched_getaffinity(0)), 16)
-        O.set_threads(cores)
-        m = MODES[args.mode]
-        v, i, c, o = scene["vertices"], scene["indices"], scene["colors"], scene["opacities"]
-        t0 = time.perf_counter()
-        fwd = O.render(v, i, c, o, W, H, 16, 16, 1 / 256, m["per_pixel_sort"], m["max_layers"])
-        t1 = time.perf_counter()
-        gi = (2.0 * (fwd["image"] - scene["target"]) / fwd["image"].size).astype(np.float32)
-        O.render_backward(gi, np.zeros((H, W), np.float32), v, i, c, o, fwd, W, H, 16, 16, m["per_pixel_sort"], m["max_layers"])
-        t2 = time.perf_counter()
-        out["cpu_baseline"] = {"value": 1.0 / (t2 - t0), "unit": "frames/s", "cores": cores, "kind": "port",
-                               "sample": f"one full forward+backward frame of the same workload (forward {t1 - t0:.2f} s, "
-                                         f"backward {t2 - t1:.2f} s), binning serial, sort/blend/backward OpenMP over tiles"}
+        single, many = cpu_oracle_baseline(scene, MODES[args.mode], W, H, cores)
+        out["cpu_baseline"] = {"value": 1.0 / many["forward_backward_seconds"], "unit": "frames/s", "cores": cores, "kind": "port",
+                               "sample": "the same frame, forward + backward: OpenMP over tiles after one warm-up, median of three "
+                                         "runs (binning, sort and ranges are serial code); the single-thread figures are one run",
+                               "openmp": many, "single_thread": dict(single, cores=1,
+                                                                     value=1.0 / single["forward_backward_seconds"])}
     print(json.dumps(out))
 
 

@@ -167,8 +167,12 @@ def forward(verts, idx, colors, opac, ids, offsets, bary_m, W, H, tw=16, th=16, 
 
 
 def backward(grad_image, grad_depthmap, verts, idx, colors, opac, ids, offsets, bary_m, fwd, W, H, tw=16, th=16,
-             per_pixel_sort=True, max_layers=32, literal=False):
-    """-> (grad_vertices (V,4), grad_colors (V,3), grad_opacities (V,)) as float64; render.cu:621-695."""
+             per_pixel_sort=True, max_layers=32, literal=False, magnitudes=False):
+    """-> (grad_vertices (V,4), grad_colors (V,3), grad_opacities (V,)) as float64; render.cu:621-695.
+
+    magnitudes: also three arrays of the same shapes with, per element, the sum of the magnitudes of everything that
+    was added into it (for a position gradient: of the products its terms are made of).  The rounding error of a
+    float32 accumulation of the same terms, in any order, is proportional to that sum, element by element."""
     suf, _ = _suf(verts.dtype)
     dt = verts.dtype
     verts, colors, opac, bary_m, grad_image, grad_depthmap = (
@@ -177,14 +181,18 @@ def backward(grad_image, grad_depthmap, verts, idx, colors, opac, ids, offsets, 
     if max_layers <= 0:
         max_layers = idx.shape[0] + 1
     V = verts.shape[0]
-    gV = np.zeros((V, 4), np.float64)
-    gC = np.zeros((V, 3), np.float64)
-    gO = np.zeros((V,), np.float64)
+    copies = 2 if magnitudes else 1
+    gV = np.zeros((copies, V, 4), np.float64)
+    gC = np.zeros((copies, V, 3), np.float64)
+    gO = np.zeros((copies, V), np.float64)
     getattr(lib(), f"tgo_backward_{suf}")(
         _p(grad_image), _p(grad_depthmap), _p(verts), _p(idx), _p(colors), _p(opac), _p(ids), _p(offsets), _p(bary_m),
         _p(_c(fwd["image"], dt)), _p(_c(fwd["depthmap"], dt)), _p(_c(fwd["weights"], dt)), _p(_c(fwd["ends"], np.int32)),
-        W, H, tw, th, int(bool(per_pixel_sort)), int(max_layers), int(bool(literal)), V, _p(gV), _p(gC), _p(gO))
-    return gV, gC, gO
+        W, H, tw, th, int(bool(per_pixel_sort)), int(max_layers), int(bool(literal)), V, _p(gV), _p(gC), _p(gO),
+        int(bool(magnitudes)))
+    if magnitudes:
+        return gV[0], gC[0], gO[0], gV[1], gC[1], gO[1]
+    return gV[0], gC[0], gO[0]
 
 
 def render(verts, idx, colors, opac, W, H, tw=16, th=16, thr=1 / 256, per_pixel_sort=True, max_layers=32):
@@ -197,9 +205,9 @@ def render(verts, idx, colors, opac, W, H, tw=16, th=16, thr=1 / 256, per_pixel_
 
 
 def render_backward(grad_image, grad_depthmap, verts, idx, colors, opac, fwd, W, H, tw=16, th=16,
-                    per_pixel_sort=True, max_layers=32, literal=False):
+                    per_pixel_sort=True, max_layers=32, literal=False, magnitudes=False):
     return backward(grad_image, grad_depthmap, verts, idx, colors, opac, fwd["sorted_ids"], fwd["offsets"], fwd["bary"],
-                    fwd, W, H, tw, th, per_pixel_sort, max_layers, literal)
+                    fwd, W, H, tw, th, per_pixel_sort, max_layers, literal, magnitudes)
 
 
 # ---- component hooks (reference src/trigrad/tests.cu:43-76) ---------------------

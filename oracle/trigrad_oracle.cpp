@@ -314,6 +314,10 @@ template <typename S> struct Scene {
     const S *verts; const int *idx; const S *colors; const S *opac;
     const int *ids; const int *offsets; const S *bary;
     int W, H, tw, th;
+    // backward pass only: > 0 makes every gradient array hold, behind its sums, the sums of the magnitudes of what was
+    // added (so many vertices further on): the scale that the rounding of a float32 accumulation of the same terms is
+    // proportional to.  Test infrastructure, not part of the reference.
+    size_t magnitudes_at = 0;
 };
 
 template <typename S> struct Frag {  // everything process_forward/backward read for one list entry
@@ -481,11 +485,10 @@ template <typename S> inline P3<S> barycentric(P2<S> v0, P2<S> v1, P2<S> v2, P2<
 
 // util.h:405-455 barycentric_backward: J[v][axis][k] = d bary_k / d vertex_v.axis, v=3 is the point.
 template <typename S>
-inline void barycentric_bwd(const S g[3], P2<S> a, P2<S> b, P2<S> c, P2<S> p, S out[4][2]) {
+inline bool barycentric_jacobian(P2<S> a, P2<S> b, P2<S> c, P2<S> p, S J[4][2][3]) {
     P3<S> l = barycentric(a, b, c, p);
     S d = a.x * (b.y - c.y) + b.x * (-a.y + c.y) + c.x * (a.y - b.y);
-    if (std::fabs(d) < eff_zero<S>()) { for (int v = 0; v < 4; v++) out[v][0] = out[v][1] = 0; return; }
-    S J[4][2][3];
+    if (std::fabs(d) < eff_zero<S>()) return false;
     J[0][0][0] = l.x * (-b.y + c.y) / d;
     J[0][0][1] = (-c.y - l.y * (b.y - c.y) + p.y) / d;
     J[0][0][2] = (b.y - l.z * (b.y - c.y) - p.y) / d;
@@ -510,7 +513,49 @@ inline void barycentric_bwd(const S g[3], P2<S> a, P2<S> b, P2<S> c, P2<S> p, S 
     J[3][1][0] = (-b.x + c.x) / d;
     J[3][1][1] = (a.x - c.x) / d;
     J[3][1][2] = (-a.x + b.x) / d;
+    return true;
+}
+template <typename S>
+inline void barycentric_bwd(const S g[3], P2<S> a, P2<S> b, P2<S> c, P2<S> p, S out[4][2]) {
+    S J[4][2][3];
+    if (!barycentric_jacobian(a, b, c, p, J)) { for (int v = 0; v < 4; v++) out[v][0] = out[v][1] = 0; return; }
     for (int v = 0; v < 4; v++)
+        for (int ax = 0; ax < 2; ax++) out[v][ax] = g[0] * J[v][ax][0] + g[1] * J[v][ax][1] + g[2] * J[v][ax][2];
+}
+// The scale of a position term (test infrastructure, not part of the reference).  A numerator such as
+// -c.y - l.y (b.y - c.y) + p.y is a small difference of screen coordinates of order one: its float32 value is
+// uncertain by 2^-24 of the SUM of its addends' magnitudes, whichever way it is evaluated (contracted into a fused
+// multiply-add or not, with l off by an ulp or not).  So every Jacobian entry is taken with the magnitudes of its
+// numerator's addends, and g with the magnitudes of the parts it is the sum of.
+template <typename S>
+inline void barycentric_bwd_magnitude(const S g[3], P2<S> a, P2<S> b, P2<S> c, P2<S> p, S out[4][2]) {
+    for (int v = 0; v < 4; v++) out[v][0] = out[v][1] = 0;
+    P3<S> l = barycentric(a, b, c, p);
+    S d = a.x * (b.y - c.y) + b.x * (-a.y + c.y) + c.x * (a.y - b.y);
+    if (std::fabs(d) < eff_zero<S>()) return;
+    const S id = 1 / std::fabs(d);
+    const auto sum3 = [&](S u, S m, S q) { return (std::fabs(u) + std::fabs(m) + std::fabs(q)) * id; };
+    const auto prod = [&](S m) { return std::fabs(m) * id; };
+    S J[3][2][3];
+    J[0][0][0] = prod(l.x * (-b.y + c.y));
+    J[0][0][1] = sum3(c.y, l.y * (b.y - c.y), p.y);
+    J[0][0][2] = sum3(b.y, l.z * (b.y - c.y), p.y);
+    J[0][1][0] = prod(l.x * (b.x - c.x));
+    J[0][1][1] = sum3(c.x, l.y * (b.x - c.x), p.x);
+    J[0][1][2] = sum3(b.x, l.z * (b.x - c.x), p.x);
+    J[1][0][0] = sum3(c.y, l.x * (a.y - c.y), p.y);
+    J[1][0][1] = prod(l.y * (a.y - c.y));
+    J[1][0][2] = sum3(a.y, l.z * (a.y - c.y), p.y);
+    J[1][1][0] = sum3(c.x, l.x * (a.x - c.x), p.x);
+    J[1][1][1] = prod(l.y * (-a.x + c.x));
+    J[1][1][2] = sum3(a.x, l.z * (a.x - c.x), p.x);
+    J[2][0][0] = sum3(b.y, l.x * (a.y - b.y), p.y);
+    J[2][0][1] = sum3(a.y, l.y * (a.y - b.y), p.y);
+    J[2][0][2] = prod(l.z * (-a.y + b.y));
+    J[2][1][0] = sum3(b.x, l.x * (a.x - b.x), p.x);
+    J[2][1][1] = sum3(a.x, l.y * (a.x - b.x), p.x);
+    J[2][1][2] = prod(l.z * (a.x - b.x));
+    for (int v = 0; v < 3; v++)
         for (int ax = 0; ax < 2; ax++) out[v][ax] = g[0] * J[v][ax][0] + g[1] * J[v][ax][1] + g[2] * J[v][ax][2];
 }
 
@@ -518,9 +563,14 @@ template <typename S> struct BackState {
     S final_alpha, alpha; S s[3] = {0, 0, 0}; S oa = 0, zoa = 0; S final_weight, final_depth;
 };
 
-inline void accum(double *p, double v) {
+// *p += v, and, if `behind` is not 0, p[behind] += magnitude (see Scene::magnitudes_at).
+inline void accum(double *p, double v, size_t behind = 0, double magnitude = 0.0) {
 #pragma omp atomic
     *p += v;
+    if (behind) {
+#pragma omp atomic
+        p[behind] += magnitude;
+    }
 }
 
 // render.cu:455-538 process_backward.  Gradients are accumulated in double: the
@@ -557,16 +607,17 @@ inline void process_backward(const Scene<S> &sc, int j, P2<S> pos, const S *gout
 
     S gb_o[3], gv_o[3], gw_o[3];
     interp_bwd_scalar(d_do, bc, sc.opac[ia], sc.opac[ib], sc.opac[ic], ws, gb_o, gv_o, gw_o);
-    for (int v = 0; v < 3; v++) accum(gO + vid[v], (double)gv_o[v]);           // :506-508
+    const size_t mag = sc.magnitudes_at;
+    for (int v = 0; v < 3; v++) accum(gO + vid[v], (double)gv_o[v], mag, std::fabs((double)gv_o[v]));  // :506-508
 
     S ao = st.alpha * o;
     S gcol[3] = {ao * gout[0], ao * gout[1], ao * gout[2]};                    // :510
     S gb_c[3], ga[3], gbv[3], gc[3], gw_c[3];
     interp_bwd_vec(gcol, bc, ca, cb, cc, ws, gb_c, ga, gbv, gc, gw_c);
     for (int k = 0; k < 3; k++) {                                              // :514-516
-        accum(gC + 3 * (size_t)ia + k, (double)ga[k]);
-        accum(gC + 3 * (size_t)ib + k, (double)gbv[k]);
-        accum(gC + 3 * (size_t)ic + k, (double)gc[k]);
+        accum(gC + 3 * (size_t)ia + k, (double)ga[k], 3 * mag, std::fabs((double)ga[k]));
+        accum(gC + 3 * (size_t)ib + k, (double)gbv[k], 3 * mag, std::fabs((double)gbv[k]));
+        accum(gC + 3 * (size_t)ic + k, (double)gc[k], 3 * mag, std::fabs((double)gc[k]));
     }
     S dd_dz = ao * gdepth / st.final_weight;                                   // :517
     if (st.final_weight < eff_zero<S>()) dd_dz = 0;
@@ -581,11 +632,20 @@ inline void process_backward(const Scene<S> &sc, int j, P2<S> pos, const S *gout
     S dxy[4][2];
     const S *va = sc.verts + 4 * (size_t)ia, *vb = sc.verts + 4 * (size_t)ib, *vc = sc.verts + 4 * (size_t)ic;
     barycentric_bwd<S>(gbary, {va[0], va[1]}, {vb[0], vb[1]}, {vc[0], vc[1]}, pos, dxy);
+    // a position term is a sum of three products that may cancel, and each of the three barycentric gradients is a sum
+    // of three parts: its scale is that of the parts, which barycentric_bwd turns into with the magnitudes as input
+    S dxy_mag[4][2] = {};
+    if (mag) {
+        S gbary_mag[3];
+        for (int k = 0; k < 3; k++) gbary_mag[k] = std::fabs(gb_o[k]) + std::fabs(gb_c[k]) + std::fabs(gb_z[k]);
+        barycentric_bwd_magnitude<S>(gbary_mag, {va[0], va[1]}, {vb[0], vb[1]}, {vc[0], vc[1]}, pos, dxy_mag);
+    }
     for (int v = 0; v < 3; v++) {                                              // :530-537
         S dw = gw_o[v] + gw_c[v] + gw_z[v];
-        accum(gV + 4 * (size_t)vid[v] + 0, (double)dxy[v][0]);
-        accum(gV + 4 * (size_t)vid[v] + 1, (double)dxy[v][1]);
-        accum(gV + 4 * (size_t)vid[v] + 3, (double)(dw + dd_dw[v]));
+        accum(gV + 4 * (size_t)vid[v] + 0, (double)dxy[v][0], 4 * mag, (double)dxy_mag[v][0]);
+        accum(gV + 4 * (size_t)vid[v] + 1, (double)dxy[v][1], 4 * mag, (double)dxy_mag[v][1]);
+        accum(gV + 4 * (size_t)vid[v] + 3, (double)(dw + dd_dw[v]), 4 * mag,
+              std::fabs((double)gw_o[v]) + std::fabs((double)gw_c[v]) + std::fabs((double)gw_z[v]) + std::fabs((double)dd_dw[v]));
     }
 }
 
@@ -660,7 +720,9 @@ template <typename S>
 void render_backward(const Scene<S> &sc, bool pps, int max_layers, int literal,
                      const S *gimage, const S *gdepthmap, const S *image, const S *depthmap, const S *weights,
                      const int *ends, int V, double *gV, double *gC, double *gO) {
-    std::fill(gV, gV + 4 * (size_t)V, 0.0); std::fill(gC, gC + 3 * (size_t)V, 0.0); std::fill(gO, gO + (size_t)V, 0.0);
+    const size_t copies = sc.magnitudes_at ? 2 : 1;  // sums, and behind them the magnitudes
+    std::fill(gV, gV + copies * 4 * (size_t)V, 0.0); std::fill(gC, gC + copies * 3 * (size_t)V, 0.0);
+    std::fill(gO, gO + copies * (size_t)V, 0.0);
     int tiles_x = (sc.W + sc.tw - 1) / sc.tw, tiles_y = (sc.H + sc.th - 1) / sc.th;
 #pragma omp parallel for schedule(dynamic, 1) num_threads(g_threads)
     for (int tile = 0; tile < tiles_x * tiles_y; tile++) {
@@ -701,8 +763,10 @@ void render_backward(const Scene<S> &sc, bool pps, int max_layers, int literal,
     extern "C" void tgo_backward_##SUF(const S *gimage, const S *gdepth, const S *v, const int *i, const S *c, const S *o, \
                                        const int *ids, const int *offsets, const S *bary, const S *image,                  \
                                        const S *depthmap, const S *weights, const int *ends, int W, int H, int tw, int th, \
-                                       int pps, int max_layers, int literal, int V, double *gV, double *gC, double *gO) {  \
+                                       int pps, int max_layers, int literal, int V, double *gV, double *gC, double *gO,    \
+                                       int magnitudes) {                                                                   \
         Scene<S> sc{v, i, c, o, ids, offsets, bary, W, H, tw, th};                                                         \
+        sc.magnitudes_at = magnitudes ? (size_t)V : 0;                                                                     \
         render_backward<S>(sc, pps != 0, max_layers, literal, gimage, gdepth, image, depthmap, weights, ends, V, gV, gC,   \
                            gO);                                                                                            \
     }                                                                                                                      \

@@ -16,7 +16,7 @@ triangle ids, image invariant under a permutation of the triangle list.
 import numpy as np
 import pytest
 
-from helpers import assert_close, to_device, u64
+from helpers import assert_gradients_close, assert_close, to_device, u64
 
 pytestmark = pytest.mark.gpu
 
@@ -115,15 +115,15 @@ def test_forward_backward_full_size(cfg, mode, cuda, oracle):
         assert_close(f"config{cfg}/{mode}: depthmap", dm[fin], fwd["depthmap"][fin], 1e-5, 1e-5)
         scale = 1.0 / fwd["image"].size if reduction == "mean" else 1.0
         gi = (2.0 * scale * (fwd["image"].astype(np.float64) - scene["target"])).astype(np.float32)
-        gV, gC, gO = oracle.render_backward(gi, zero_gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"],
-                                            fwd, W, H, 16, 16, m["per_pixel_sort"], m["max_layers"])
-        for label, g, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
+        wanted = oracle.render_backward(gi, zero_gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"],
+                                        fwd, W, H, 16, 16, m["per_pixel_sort"], m["max_layers"], magnitudes=True)
+        for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), (v.grad, c.grad, o.grad), wanted[:3], wanted[3:]):
             g = g.cpu().numpy()
-            if reduction == "mean":
+            if reduction == "mean":  # the benchmark's loss: gradients around 1e-7, the stated bar as it is
                 assert_close(f"config{cfg}/{mode}/mean: {label}", g, w, 1e-4, 1e-6)
-            else:
-                # float32 atomics in arbitrary order against the float64 sum of the same terms
-                assert_close(f"config{cfg}/{mode}/sum: {label}", g, w, 1e-4, 1e-6 * max(1.0, float(np.abs(w).max())))
+            # float32 atomics in arbitrary order against the float64 sum of the same terms: the stated bar plus the
+            # rounding of a float32 sum of the element's own terms
+            assert_gradients_close(f"config{cfg}/{mode}/{reduction}: {label}", g, w, mag)
         del v, c, o, image, depthmap, loss, diff
     torch.cuda.empty_cache()
 

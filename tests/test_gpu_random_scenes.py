@@ -4,8 +4,8 @@ test_gpu_render, against the oracle on the same inputs."""
 import numpy as np
 import pytest
 
-from helpers import assert_close
-from test_gpu_render import GRAD_ATOL, GRAD_RTOL, _check_forward, _forward_both, _grad_inputs
+from helpers import assert_gradients_close
+from test_gpu_render import _check_forward, _forward_both, _grad_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -33,12 +33,10 @@ def test_random_scenes_match_oracle(block, cuda, oracle):
         _check_forward(name, want, got)
         gi, gd = _grad_inputs(scene, case, bool(rng.integers(0, 2)))
         wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
-                                        W, H, tw, th, pps, ml, literal=False)
+                                        W, H, tw, th, pps, ml, literal=False, magnitudes=True)
         image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
         out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                                  d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H,
                                  tw, th, thr, pps, ml, resume=resume)
-        for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, wanted):
-            scale = float(np.nanmax(np.abs(w))) if w.size else 0.0
-            assert_close(f"{name}: {label}", np.nan_to_num(g.cpu().numpy().astype(np.float64)), np.nan_to_num(w), GRAD_RTOL,
-                         GRAD_ATOL + 2e-6 * scale)
+        for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, wanted[:3], wanted[3:]):
+            assert_gradients_close(f"{name}: {label}", g.cpu().numpy(), w, mag)

@@ -12,13 +12,12 @@ Everything here calls the C ABI of libtrigrad_hip.so through trigrad_amd.
 import numpy as np
 import pytest
 
-from helpers import assert_close, to_device, u64
+from helpers import GRAD_ATOL, GRAD_RTOL, assert_gradients_close, assert_close, to_device, u64
 from test_gpu_stages import SCENES
 
 pytestmark = pytest.mark.gpu
 
 IMAGE_ATOL = 1e-5
-GRAD_RTOL, GRAD_ATOL = 1e-4, 1e-6
 
 MODES = {
     "A_default": dict(per_pixel_sort=True, max_layers=32),
@@ -116,15 +115,14 @@ def test_tile_list_longer_than_16_bit_positions(mode, tile, cuda, oracle):
     assert lengths.max() > 65535 and (tile == 32 or lengths.min() < 65535)
     _check_forward(f"long list/{mode}", want, got)
     gi, gd = _grad_inputs(scene, 9, True)
-    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
-                                        32, 32, tile, tile, m["per_pixel_sort"], ml, literal=False)
+    wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                    32, 32, tile, tile, m["per_pixel_sort"], ml, literal=False, magnitudes=True)
     image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
     out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                              d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, 32, 32,
                              tile, tile, 1 / 256, m["per_pixel_sort"], ml, resume=resume)
-    for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
-        scale = float(np.abs(w).max())
-        assert_close(f"long list/{mode}: {label}", g.cpu().numpy().astype(np.float64), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * scale)
+    for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, wanted[:3], wanted[3:]):
+        assert_gradients_close(f"long list/{mode}: {label}", g.cpu().numpy(), w, mag)
 
 
 def _grad_inputs(scene, seed, with_depth):
@@ -136,7 +134,8 @@ def _grad_inputs(scene, seed, with_depth):
 
 
 BACKWARD_SCENES = ["config0", "soup_varying_w", "soup_shared", "soup_big_tris", "soup_tile4", "soup_tile32", "soup_tile_8x4",
-                   "squares", "large_triangles", "depth_overlap", "unit_square_negative_z", "grid_mesh", "degenerate", "center_island", "soup_tile8", "soup_tile_24x16"]
+                   "squares", "large_triangles", "depth_overlap", "overlapping_triangles", "unit_square_negative_z", "overlap_mesh_inf_w",
+                   "grid_mesh", "degenerate", "center_island", "soup_tile8", "soup_tile_24x16"]
 
 
 @pytest.mark.parametrize("with_depth", [False, True])
@@ -150,8 +149,8 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
     d, want, got, ml = _forward_both(scene, tw, th, m, cuda, oracle)
     W, H = scene["width"], scene["height"]
     gi, gd = _grad_inputs(scene, 5, with_depth)
-    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
-                                        W, H, tw, th, m["per_pixel_sort"], ml, literal=False)
+    wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                    W, H, tw, th, m["per_pixel_sort"], ml, literal=False, magnitudes=True)
     image, depthmap, weights, sorted_ids, offsets, bary, ends, _, resume = got
     # the blend order is saved exactly when per-pixel order meets max_layers <= 32;
     # then the route that selects the fragments again is checked as well
@@ -167,14 +166,8 @@ def test_backward_matches_oracle(name, mode, with_depth, cuda, oracle):
         out = _C.render_backward(torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda), d["vertices"], d["indices"],
                                  d["colors"], d["opacities"], sorted_ids, offsets, bary, image, depthmap, weights, ends, W, H,
                                  tw, th, 1 / 256, m["per_pixel_sort"], ml, resume=res)
-        for label, g, w in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, (gV, gC, gO)):
-            g = g.cpu().numpy().astype(np.float64)
-            # float32 summation of n terms: allow rtol on the result plus the rounding
-            # of the largest partial sums (scale of the gradient array)
-            scale = float(np.nanmax(np.abs(w))) if w.size else 0.0
-            assert_close(f"{name}/{mode}{route}: {label}", np.nan_to_num(g), np.nan_to_num(w), GRAD_RTOL,
-                         GRAD_ATOL + 2e-6 * scale)
-            assert np.array_equal(np.isnan(g), np.isnan(w))
+        for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), out, wanted[:3], wanted[3:]):
+            assert_gradients_close(f"{name}/{mode}{route}: {label}", g.cpu().numpy(), w, mag)  # NaN where the oracle has NaN
         assert float(out[0][:, 2].abs().max()) == 0.0  # z never receives a gradient (render.cu:531-533)
     if name == "soup_shared" and with_depth:
         # the three layouts of the gradient arrays the kernels know: dense, one (V,8) block, run-time strides
@@ -222,10 +215,10 @@ def test_render_autograd_end_to_end(cuda, oracle):
                             max_layers=ml)
         assert_close("image", image.detach().cpu().numpy(), fwd["image"], 0.0, IMAGE_ATOL)
         gi = 2.0 * (fwd["image"] - scene["target"])
-        gV, gC, gO = oracle.render_backward(gi, np.zeros((H, W), np.float32), scene["vertices"], scene["indices"], scene["colors"],
-                                            scene["opacities"], fwd, W, H, per_pixel_sort=pps, max_layers=ml)
-        for label, g, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
-            assert_close(label, g.cpu().numpy(), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * float(np.abs(w).max()))
+        wanted = oracle.render_backward(gi, np.zeros((H, W), np.float32), scene["vertices"], scene["indices"], scene["colors"],
+                                        scene["opacities"], fwd, W, H, per_pixel_sort=pps, max_layers=ml, magnitudes=True)
+        for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), (v.grad, c.grad, o.grad), wanted[:3], wanted[3:]):
+            assert_gradients_close(label, g.cpu().numpy(), w, mag)
 
 
 def test_loss_on_depth_only(cuda, oracle):
@@ -245,10 +238,10 @@ def test_loss_on_depth_only(cuda, oracle):
     (torch.where(hit, depthmap, torch.zeros_like(depthmap)) * weight).sum().backward()
     fwd = oracle.render(scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], W, H)
     gd = np.where(np.isfinite(fwd["depthmap"]), weight.cpu().numpy(), 0.0).astype(np.float32)
-    gV, gC, gO = oracle.render_backward(np.zeros((H, W, 4), np.float32), gd, scene["vertices"], scene["indices"], scene["colors"],
-                                        scene["opacities"], fwd, W, H)
-    for label, g, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
-        assert_close(label, g.cpu().numpy(), w, GRAD_RTOL, GRAD_ATOL + 2e-6 * float(np.abs(w).max()))
+    wanted = oracle.render_backward(np.zeros((H, W, 4), np.float32), gd, scene["vertices"], scene["indices"], scene["colors"],
+                                    scene["opacities"], fwd, W, H, magnitudes=True)
+    for label, g, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), (v.grad, c.grad, o.grad), wanted[:3], wanted[3:]):
+        assert_gradients_close(label, g.cpu().numpy(), w, mag)
     assert float(v.grad.abs().max()) > 0
 
 
@@ -453,10 +446,10 @@ def test_native_surface_as_the_reference_wrapper_calls_it(mode, drop_private_sta
     finite = np.isfinite(want["depthmap"])
     gd = np.where(finite, gd, 0).astype(np.float32)
     torch.autograd.backward([image, depthmap], [torch.from_numpy(gi).to(cuda), torch.from_numpy(gd).to(cuda)])
-    gV, gC, gO = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
-                                        W, H, 16, 16, m["per_pixel_sort"], ml)
-    for label, got, w in (("grad_vertices", v.grad, gV), ("grad_colors", c.grad, gC), ("grad_opacities", o.grad, gO)):
-        assert_close(f"{mode}: {label}", got.cpu().numpy(), w, 1e-4, 1e-6 + 2e-6 * float(np.abs(w).max()))
+    wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
+                                    W, H, 16, 16, m["per_pixel_sort"], ml, magnitudes=True)
+    for label, got, w, mag in zip(("grad_vertices", "grad_colors", "grad_opacities"), (v.grad, c.grad, o.grad), wanted[:3], wanted[3:]):
+        assert_gradients_close(f"{mode}: {label}", got.cpu().numpy(), w, mag)
     # the attribute on `ends` must survive save_for_backward, or every backward pass pays for a second forward kernel
     assert Fn.resume_seen == [not drop_private_state]
 

@@ -27,6 +27,7 @@ def _scenes():
         "squares": lambda: (S.overlapping_squares(10), 4, 4),
         "large_triangles": lambda: (S.large_triangles(3, r=4), 4, 4),
         "depth_overlap": lambda: (S.depth_overlap(), 16, 16),
+        "overlapping_triangles": lambda: (S.overlapping_triangles(), 16, 16),
         "unit_square_negative_z": lambda: (S.unit_square(), 16, 16),
         "overlap_mesh_inf_w": lambda: (S.overlap_mesh(), 16, 16),
         "grid_mesh": lambda: (S.grid_mesh(40, 40, -0.9, 0.9, -0.9, 0.9, width=96, height=96), 16, 16),
