@@ -155,6 +155,30 @@ def test_split_clipped_empty_and_gradients():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_split_clipped_on_the_device_matches_triangle_loop(seed, cuda):
+    """The same comparison with the tensors on the GPU: split_clipped's stable argsort, nonzero and gathers run as
+    device kernels there (notebooks/renderer.ipynb cell 15 runs it on cuda tensors too)."""
+    cv, idx, col, op = _mesh(seed)
+    counts = ((cv[idx][:, :, 2] + cv[idx][:, :, 3]) >= 0).sum(axis=1)
+    assert set(counts.tolist()) == {0, 1, 2, 3}
+    v, i, c, o = camera.split_clipped(*(torch.from_numpy(a).to(cuda) for a in (cv, idx, col, op)))
+    assert v.device.type == "cuda" and i.device.type == "cuda" and i.dtype == torch.int32
+    wv, wc, wo = _split_loop(cv, idx, col, op)
+    n = int((counts == 3).sum() + (counts == 1).sum() + 2 * (counts == 2).sum())
+    np.testing.assert_array_equal(i.cpu().numpy(), np.arange(3 * n).reshape(n, 3))
+    np.testing.assert_allclose(v.cpu().numpy(), wv, rtol=0, atol=1e-14)
+    np.testing.assert_allclose(c.cpu().numpy(), wc, rtol=0, atol=1e-14)
+    np.testing.assert_allclose(o.cpu().numpy(), wo, rtol=0, atol=1e-14)
+    # and in the renderer's precision, against the float64 loop
+    v32, i32, c32, o32 = camera.split_clipped(*(torch.from_numpy(a.astype(np.float32) if a.dtype == np.float64 else a).to(cuda)
+                                                for a in (cv, idx, col, op)))
+    assert v32.dtype == torch.float32 and v32.shape == (3 * n, 4)
+    np.testing.assert_allclose(v32.cpu().numpy(), wv, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(c32.cpu().numpy(), wc, rtol=2e-5, atol=2e-5)
+
+
+@pytest.mark.gpu
 def test_projected_split_mesh_renders(cuda):
     """A mesh reaching behind the camera renders to finite values after splitting, and
     splitting a mesh that lies wholly in front changes nothing in the image."""

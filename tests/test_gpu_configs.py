@@ -142,3 +142,37 @@ def test_image_invariant_under_triangle_permutation(cfg, cuda):
     perm = torch.randperm(d["indices"].shape[0], device=cuda, generator=torch.Generator(device=cuda).manual_seed(0))
     b, _ = trigrad_amd.render(d["vertices"], d["indices"][perm].contiguous(), d["colors"], d["opacities"], W, H)
     assert float((a - b).abs().max()) <= 1e-5
+
+
+def test_stage_timings_describe_the_frame_that_runs(cuda):
+    """record_timing=True times the route an untimed call runs (the same entry points in the same order, with the
+    reference's five stage names, render.cu:723-747): on the headline frame the stage times add up to the forward time
+    of an untimed call within a tenth."""
+    import torch
+    import trigrad_amd
+    scene = _scene(2)
+    W, H = scene["width"], scene["height"]
+    d = to_device({k: scene[k] for k in ("vertices", "indices", "colors", "opacities")}, cuda)
+    args = (d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, 16, 16, 1 / 256)
+    kinds = {}
+    for pps, ml in ((False, -1), (True, 32)):
+        for _ in range(3):
+            trigrad_amd.render(*args, False, pps, ml)
+        untimed = []
+        for _ in range(7):
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            trigrad_amd.render(*args, False, pps, ml)
+            e1.record()
+            e1.synchronize()
+            untimed.append(e0.elapsed_time(e1) / 1000.0)
+        sums = []
+        for _ in range(7):
+            torch.cuda.synchronize()
+            _, _, timings = trigrad_amd.render(*args, True, pps, ml)
+            assert set(timings) == {"init", "per_tile_lists", "sorting", "bary_transforms", "rasterization"}
+            sums.append(sum(timings.values()))
+        a, b = float(np.median(untimed)), float(np.median(sums))
+        kinds[pps] = (a, b)
+        assert abs(b - a) <= 0.1 * a, f"per_pixel_sort={pps}: stages add up to {b * 1e3:.3f} ms, an untimed forward pass takes {a * 1e3:.3f} ms"
