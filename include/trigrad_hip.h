@@ -110,7 +110,8 @@ int tg_scan_exclusive_u32(const uint32_t *in, uint32_t *out, int64_t n, uint32_t
  * reference: it is for callers that cannot allocate device memory or pass a
  * workspace (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  The look-back state lives in a device array inside
- * the library (64 KiB per GPU, held until the process ends) instead of a
+ * the library (65 600 bytes per GPU: 64 for the ticket, 8 for each of 8192 tiles
+ * of 2048 elements; held until the process ends) instead of a
  * workspace; the call allocates and frees nothing.  n may not exceed
  * TG_SCAN_NOALLOC_MAX_N = tg_scan_noalloc_max_n() (TG_E_ARG otherwise).  All
  * calls on one GPU share that array: calls that overlap on one GPU (two

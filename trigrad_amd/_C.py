@@ -3,10 +3,12 @@ pybind module (src/trigrad/module.cu:8-21, render.h) with the same names and
 argument order, implemented by calling the C ABI of libtrigrad_hip.so on the
 current torch stream.  torch is used for device memory and streams only.
 
-`render_forward` runs the key pipeline the library is built around:
-    bin_count -> scan -> (read K) -> bin_emit -> sort_pairs -> tile_ranges
-    -> cartesian_to_bary -> forward kernel
-and the individual stages are exposed as functions for tests and benchmarks.
+`render_forward` runs the frame's route:
+    bin_frame (count + scan, then key emission that reads K on the device) -> (K to the host, bary matrices meanwhile)
+    -> build_frame_lists (two passes over the tile bits through memory, depth bits and tile ranges per tile)
+    -> forward kernel
+The double build and frames with more than 2^21 tiles go through bin_setup + build_tile_lists, and the single stages
+(bin_count, scan_exclusive, bin_emit, sort_pairs, tile_ranges) are exposed as functions for tests and benchmarks.
 """
 import ctypes as C
 import threading

@@ -1,14 +1,16 @@
-// tg_binning.hip -- tile binning (count, key emission) and bary matrices.
+// tg_binning.hip -- tile binning (count, scan, key emission) and bary matrices.
 //
-// count and bary are HBM-bound streaming kernels; emit is bound by the
-// clipping arithmetic it does per key:
-//   count   reads 12 B indices + 3 x 16 B vertex gathers, writes 4 B per triangle
-//   emit    one thread per KEY (not per triangle), so a triangle that covers
-//           thousands of tiles is spread over thousands of lanes; reads the
-//           triangle again (L2 hits for neighbouring keys), clips it to the
-//           tile (polygon in LDS), writes 8 B key + 4 B payload per key,
-//           coalesced
-//   bary    reads 60 B, writes 36 B per triangle
+// Three routes to the same keys, all with one thread per KEY in the emission (a triangle that covers thousands of
+// tiles is spread over thousands of lanes) and the clip polygon of a key in LDS:
+//   stage by stage   bin_count_kernel (12 B indices + 3 x 16 B vertex gathers read, 4 B written per triangle), the
+//                    scan of tg_scan.hip, bin_emit_kernel (reads the triangle again, 12 B written per key)
+//   two calls        bin_setup_kernel (count + scan + a 48-byte record per triangle in one pass), then
+//                    bin_emit_records_kernel from the records; the host reads K in between
+//   one call         frame_scan_kernel + frame_emit_kernel: as the two calls, with nothing to clear beforehand,
+//                    the digit totals of the sort from two additions per triangle, K read on the device, and only
+//                    the clip passes run that a key needs
+// The count + scan kernels and bary_kernel (60 B read, 36 B written per triangle) are bound by memory traffic, the
+// emission kernels by the vector instructions of the clipping.
 #include "tg_raster.hpp"
 #include "tg_scan.hpp"
 #include "tg_sort_plan.hpp"

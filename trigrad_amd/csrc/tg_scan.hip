@@ -161,13 +161,16 @@ constexpr size_t kStaticScanBytes = 64 + (size_t)(kStaticScanMaxN / kScanTile) *
 static_assert(kStaticScanMaxN % kScanTile == 0, "whole tiles");
 static __device__ __align__(256) unsigned char scratch[kStaticScanBytes];
 
-static void *static_scan_workspace() {
+// -> the array's address on the current device, or nullptr with *error = the runtime's error code.
+static void *static_scan_workspace(int *error) {
     static std::mutex mutex;
     static void *address[kMaxDevices] = {nullptr};
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    const hipError_t have_device = hipGetDevice(&dev);
+    if (have_device != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
         set_error("tg_scan_exclusive_u32_noalloc: no current device");
+        *error = have_device != hipSuccess ? (int)have_device : (int)hipErrorInvalidDevice;
         return nullptr;
     }
     std::lock_guard<std::mutex> lock(mutex);
@@ -177,6 +180,7 @@ static void *static_scan_workspace() {
         if (e != hipSuccess || !ptr) {
             (void)hipGetLastError();
             set_error("tg_scan_exclusive_u32_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            *error = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
             return nullptr;
         }
         address[dev] = ptr;
@@ -193,8 +197,9 @@ extern "C" int tg_scan_exclusive_u32_noalloc(const uint32_t *in, uint32_t *out, 
                   "use tg_scan_exclusive_u32 with a workspace", (long long)n, (long long)kStaticScanMaxN);
         return TG_E_ARG;
     }
-    void *workspace = static_scan_workspace();
-    if (!workspace) return TG_E_ARG;
+    int runtime_error = 0;
+    void *workspace = static_scan_workspace(&runtime_error);
+    if (!workspace) return runtime_error;  // a hipError_t: the arguments were not at fault
     return scan_run("tg_scan_exclusive_u32_noalloc", in, out, n, total, workspace, status, head_stride, head_capacity, heads,
                     (hipStream_t)stream);
 }
