@@ -294,12 +294,14 @@ int tg_list_bounds(const tg_real *vertices, int32_t n_vertices, const int32_t *i
  * blended entry, and last_depth (H,W) = that entry's pixel depth when
  * per_pixel_sort is on (render.cu:605-606 lastJ / lastDepth).  last and
  * last_depth may be NULL; the backward pass needs them.
- * fragments (max_layers,H,W) int32, or NULL: with per_pixel_sort and
+ * fragments (2*max_layers,H,W) uint16, or NULL: with per_pixel_sort and
  * max_layers <= TG_MAX_SAVED_LAYERS the kernel also writes, for every pixel,
  * the list positions (relative to the tile's start) of its blended fragments
- * in blend order (layer k of pixel p at fragments[k*H*W + p], k < ends[p]);
- * tg_render_backward then walks them backwards instead of selecting the
- * fragments again (the reference re-selects, render.cu:667-693).
+ * in blend order: the low 16 bits of layer k of pixel p at fragments[k*H*W + p],
+ * k < ends[p], and, only in tiles whose list holds more than 65535 entries, the
+ * high 16 bits at fragments[(max_layers + k)*H*W + p] (elsewhere that half is
+ * left as it was).  tg_render_backward then walks them backwards instead of
+ * selecting the fragments again (the reference re-selects, render.cu:667-693).
  * hit_masks (tg_hit_mask_words() uint64 words), or NULL: without per_pixel_sort
  * the kernel also writes, for every pixel and every 64 consecutive entries of
  * its tile's list that it looked at, which of them cover the pixel, and per
@@ -316,7 +318,7 @@ int tg_render_forward(const tg_real *vertices, const int32_t *indices, const tg_
                       const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, int width, int height,
                       int tile_w, int tile_h, tg_real early_stopping_threshold, int per_pixel_sort, int max_layers,
                       tg_real *image, tg_real *depthmap, tg_real *final_weights, int32_t *ends, int32_t *last,
-                      tg_real *last_depth, int32_t *fragments, uint64_t *hit_masks,
+                      tg_real *last_depth, uint16_t *fragments, uint64_t *hit_masks,
                       const tg_real *batch_bounds, const int32_t *far_start, const uint32_t *list_status, void *stream);
 
 /* ---- (5) backward ----------------------------------------------------------- */
@@ -336,7 +338,7 @@ int tg_render_backward(const tg_real *grad_image, const tg_real *grad_depthmap, 
                        const int32_t *indices, const tg_real *colors, const tg_real *opacities,
                        const int32_t *sorted_ids, const int32_t *offsets, const tg_real *bary, const tg_real *image,
                        const tg_real *depthmap, const tg_real *final_weights, const int32_t *ends, const int32_t *last,
-                       const tg_real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width, int height,
+                       const tg_real *last_depth, const uint16_t *fragments, const uint64_t *hit_masks, int width, int height,
                        int tile_w, int tile_h,
                        tg_real early_stopping_threshold, int per_pixel_sort, int max_layers, tg_real *grad_vertices,
                        tg_real *grad_colors, tg_real *grad_opacities, int vertex_stride, int color_stride,

@@ -30,7 +30,7 @@ def test_random_scenes_match_oracle(block, cuda, oracle):
         thr = float(rng.choice([1 / 256, 0.0, 0.05, 0.5]))
         name = f"case {case}: {W}x{H}, tiles {tw}x{th}, {n} triangles of {sigma} px, {mode}, threshold {thr}"
         d, want, got, ml = _forward_both(scene, tw, th, mode, cuda, oracle, thr=thr)
-        _check_forward(name, want, got)
+        _check_forward(name, want, got, (th, tw))
         gi, gd = _grad_inputs(scene, case, bool(rng.integers(0, 2)))
         wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
                                         W, H, tw, th, pps, ml, literal=False, magnitudes=True)

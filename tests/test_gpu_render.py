@@ -46,7 +46,8 @@ def _forward_both(scene, tw, th, mode, cuda, oracle, thr=1 / 256):
     return d, want, got, ml
 
 
-def _check_forward(name, want, got):
+def _check_forward(name, want, got, tile_shape):
+    from trigrad_amd import _C
     image, depthmap, weights, sorted_ids, offsets, bary, ends, timings, (last, last_depth, status, fragments, hit_masks) = got
     status.verify()
     np.testing.assert_array_equal(offsets.cpu().numpy(), want["offsets"])
@@ -64,7 +65,8 @@ def _check_forward(name, want, got):
     if fragments is not None:
         # saved blend order: `ends` valid layers per pixel, no list position twice, and the last
         # layer is the entry `last` points at (the backward parity tests check the content)
-        fr = fragments.cpu().numpy()
+        tile_h, tile_w = tile_shape
+        fr = _C.saved_blend_order(fragments, offsets, tile_w, tile_h).cpu().numpy()
         en, la = want["ends"], want["last"]
         layer = np.arange(fr.shape[0])[:, None, None]
         valid = layer < en[None]
@@ -84,7 +86,7 @@ def _check_forward(name, want, got):
 def test_forward_matches_oracle(name, mode, cuda, oracle):
     scene, tw, th = SCENES[name]()
     _, want, got, _ = _forward_both(scene, tw, th, MODES[mode], cuda, oracle)
-    _check_forward(f"{name}/{mode}", want, got)
+    _check_forward(f"{name}/{mode}", want, got, (th, tw))
 
 
 def _long_list_scene():
@@ -113,7 +115,7 @@ def test_tile_list_longer_than_16_bit_positions(mode, tile, cuda, oracle):
     lengths = np.diff(want["offsets"])
     # 16x16: one long list next to short ones; 32x32: the one tile is four workgroups on the long list
     assert lengths.max() > 65535 and (tile == 32 or lengths.min() < 65535)
-    _check_forward(f"long list/{mode}", want, got)
+    _check_forward(f"long list/{mode}", want, got, (tile, tile))
     gi, gd = _grad_inputs(scene, 9, True)
     wanted = oracle.render_backward(gi, gd, scene["vertices"], scene["indices"], scene["colors"], scene["opacities"], want,
                                     32, 32, tile, tile, m["per_pixel_sort"], ml, literal=False, magnitudes=True)

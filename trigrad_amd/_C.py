@@ -88,7 +88,7 @@ def bin_count(vertices, indices, width, height, tile_width, tile_height):
 OWNER_STRIDE = 256  # keys per workgroup of the emission kernel
 MAX_SAVED_LAYERS = 32  # TG_MAX_SAVED_LAYERS of the C header
 # With per_pixel_sort and max_layers <= MAX_SAVED_LAYERS the forward pass saves every pixel's
-# blend order ((max_layers, H, W) int32) and the backward pass walks it in reverse instead of
+# blend order (16-bit planes, see saved_blend_order) and the backward pass walks it in reverse instead of
 # selecting the fragments again.  False trades the memory for the re-selection.
 SAVE_BLEND_ORDER = True
 # Without per_pixel_sort the forward pass saves which list entries cover which pixel (one bit per pair it
@@ -313,6 +313,19 @@ def build_tile_lists(setup, n_keys, emit_only=False, prepared=None):
 _frame_states = {}  # device index -> dict(frame, epoch): the state tg_bin_frame keeps between calls
 _frame_lock = threading.Lock()
 _FRAME_TAIL = 256  # bytes behind the library's frame state: K and the status word of the binning
+
+
+def saved_blend_order(fragments, offsets, tile_width, tile_height):
+    """(max_layers, H, W) int32 list positions, relative to the tile's start, out of the planes the forward pass
+    saved: the low halves in the first max_layers planes, the high halves (written only in tiles whose list holds
+    more than 65535 entries) in the rest.  Layer k of a pixel means something for k < ends only."""
+    layers, height, width = fragments.shape[0] // 2, fragments.shape[1], fragments.shape[2]
+    tiles_x, tiles_y = -(-width // tile_width), -(-height // tile_height)
+    lengths = (offsets[1:] - offsets[:-1]).reshape(tiles_y, tiles_x)
+    is_long = (lengths > 0xFFFF).repeat_interleave(tile_height, 0).repeat_interleave(tile_width, 1)[:height, :width]
+    low = fragments[:layers].to(torch.int32) & 0xFFFF
+    high = fragments[layers:].to(torch.int32) & 0xFFFF
+    return torch.where(is_long[None], low | (high << 16), low)
 
 
 def bin_frame_supported(vertices, width, height, tile_width, tile_height):
@@ -584,7 +597,7 @@ def _forward_full(vertices, indices, colors, opacities, width, height, tile_widt
         last = torch.empty((height, width), dtype=torch.int32, device=dev)
         last_depth = torch.empty((height, width), dtype=real, device=dev) if per_pixel_sort else None
         save_order = bool(per_pixel_sort) and SAVE_BLEND_ORDER and 0 < int(max_layers) <= MAX_SAVED_LAYERS
-        fragments = torch.empty((int(max_layers), height, width), dtype=torch.int32, device=dev) if save_order else None
+        fragments = torch.empty((2 * int(max_layers), height, width), dtype=torch.int16, device=dev) if save_order else None
 
         timer.start("per_tile_lists")
         T = num_tiles(width, height, tile_width, tile_height)
@@ -694,7 +707,7 @@ def _resume_by_forward(vertices, indices, colors, opacities, sorted_ids, offsets
     last = torch.empty((height, width), dtype=torch.int32, device=dev)
     last_depth = torch.empty((height, width), dtype=real, device=dev) if per_pixel_sort else None
     save_order = bool(per_pixel_sort) and SAVE_BLEND_ORDER and 0 < int(max_layers) <= MAX_SAVED_LAYERS
-    fragments = torch.empty((int(max_layers), height, width), dtype=torch.int32, device=dev) if save_order else None
+    fragments = torch.empty((2 * int(max_layers), height, width), dtype=torch.int16, device=dev) if save_order else None
     hit_masks = None
     if not per_pixel_sort and SAVE_HIT_MASKS:
         words = int(lib.tg_hit_mask_words(sorted_ids.numel(), width, height, tile_width, tile_height))

@@ -31,7 +31,7 @@ struct BackwardArgs {
     const int32_t *ends;
     const int32_t *last;
     const real *last_depth;
-    const int32_t *fragments;  // saved by the forward pass, or null
+    const uint16_t *fragments;  // saved by the forward pass (low halves, then high halves for long lists), or null
     const uint64_t *hit_masks; // saved by the tile-order forward pass, or null
     real *grad_vertices;
     real *grad_colors;
@@ -835,7 +835,13 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
         n = min(g.ends[p.index], a.max_layers);  // render.cu:642
     }
     const int64_t plane = (int64_t)a.W * a.H;
-    auto position_of_step = [&](int s) { return (s < n) ? g.fragments[(int64_t)(n - 1 - s) * plane + p.index] : 0; };
+    const bool long_list = end - start > 0xffff;  // then the positions' high halves were saved as well
+    auto position_of_step = [&](int s) {
+        if (s >= n) return 0;
+        const int64_t at = (int64_t)(n - 1 - s) * plane + p.index;
+        const int low = g.fragments[at];
+        return long_list ? low | ((int)g.fragments[(int64_t)a.max_layers * plane + at] << 16) : low;
+    };
     // the list positions of my next four steps
     int ahead0 = position_of_step(0), ahead1 = position_of_step(1), ahead2 = position_of_step(2), ahead3 = position_of_step(3);
     const int total = __builtin_amdgcn_readlane((int)wave_inclusive_scan_u32((uint32_t)n), kWave - 1);
@@ -971,7 +977,7 @@ extern "C" int tg_render_backward(const real *grad_image, const real *grad_depth
                                   const int32_t *indices, const real *colors, const real *opacities,
                                   const int32_t *sorted_ids, const int32_t *offsets, const real *bary, const real *image,
                                   const real *depthmap, const real *final_weights, const int32_t *ends, const int32_t *last,
-                                  const real *last_depth, const int32_t *fragments, const uint64_t *hit_masks, int width,
+                                  const real *last_depth, const uint16_t *fragments, const uint64_t *hit_masks, int width,
                                   int height, int tile_w,
                                   int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers, real *grad_vertices,
                                   real *grad_colors, real *grad_opacities, int vertex_stride, int color_stride,

@@ -506,7 +506,7 @@ __global__ __launch_bounds__(kBinThreads) void bin_emit_records_kernel(const rea
 // it.  So a pass is left out only when the bounds clear the tile edge by that margin, and is run, with its own
 // test of every vertex, whenever they do not: the polygon is the reference's in every case.
 constexpr int kEmitThreads = 256;
-constexpr int kEmitWaves = kEmitThreads / kWave;
+[[maybe_unused]] constexpr int kEmitWaves = kEmitThreads / kWave;
 constexpr int kEmitKeys = 2;  // keys per thread
 constexpr int kEmitChunk = kEmitThreads * kEmitKeys;
 constexpr int kFrameMaxTiles = 1 << 21;  // the reciprocal multiply finds a key's column exactly up to here

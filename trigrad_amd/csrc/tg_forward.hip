@@ -23,7 +23,10 @@ struct ForwardOut {
     int32_t *ends;
     int32_t *last;
     real *last_depth;
-    int32_t *fragments;  // (max_layers, H, W): list positions, relative to the tile's start, in blend order; may be null
+    // Blend order, may be null: 2 * max_layers planes of H * W 16-bit words.  Plane l holds the low half of the
+    // list position (relative to the tile's start) of every pixel's layer l; plane max_layers + l the high half,
+    // written and read only in tiles whose list is longer than kShortList.
+    uint16_t *fragments;
     uint64_t *hit_masks; // tile order: which list entries cover which pixel, 64 entries per word (see hit_mask_chunk); may be null
     const uint32_t *list_status;  // status word of the kernels that made the lists (TG_STATUS_*); may be null
 };
@@ -287,7 +290,13 @@ __device__ __forceinline__ void pixel_order_tile(const RasterArgs &a, const Forw
                         real b0, b1, b2;
                         bary_apply(r[u].m, p.px, p.py, b0, b1, b2);
                         if (!bary_inside(b0, b1, b2)) continue;  // cannot happen: the selection tested it
-                        if (out.fragments) out.fragments[(int64_t)s.blended * ((int64_t)a.W * a.H) + p.index] = tk.j(i0 + u);
+                        if (out.fragments) {
+                            const int64_t plane = (int64_t)a.W * a.H, at = (int64_t)s.blended * plane + p.index;
+                            const int rel = tk.j(i0 + u);
+                            out.fragments[at] = (uint16_t)rel;
+                            if (sizeof(Pos) > sizeof(uint16_t) && end - start > kShortList)
+                                out.fragments[(int64_t)a.max_layers * plane + at] = (uint16_t)(rel >> 16);
+                        }
                         blend_fragment(s, r[u], b0, b1, b2);
                     }
                 }
@@ -416,7 +425,7 @@ extern "C" int tg_render_forward(const real *vertices, const int32_t *indices, c
                                  const int32_t *sorted_ids, const int32_t *offsets, const real *bary, int width, int height,
                                  int tile_w, int tile_h, real early_stopping_threshold, int per_pixel_sort, int max_layers,
                                  real *image, real *depthmap, real *final_weights, int32_t *ends, int32_t *last,
-                                 real *last_depth, int32_t *fragments, uint64_t *hit_masks, const real *batch_bounds,
+                                 real *last_depth, uint16_t *fragments, uint64_t *hit_masks, const real *batch_bounds,
                                  const int32_t *far_start, const uint32_t *list_status, void *stream) {
     if (int e = check_raster_args("tg_render_forward", width, height, tile_w, tile_h, max_layers)) return e;
     if (!vertices || !indices || !colors || !opacities || !offsets || !bary || !image || !depthmap || !final_weights || !ends) {
