@@ -53,6 +53,16 @@ struct alignas(16) BackRecord {
 constexpr int kBackReals = 36;  // scalars in front of the ids
 static_assert(offsetof(BackRecord, id) == kBackReals * sizeof(real), "BackRecord layout");
 
+// 1 / x to within one unit in the last place: the hardware estimate and one Newton step where
+// the estimate is an ordinary number (zero, infinity and NaN pass through as they are).  Used
+// where the reference divides in its backward pass and the quotient is no carried state.
+__device__ __forceinline__ float reciprocal(float x) {
+    const float r = __builtin_amdgcn_rcpf(x);
+    const float refined = __builtin_fmaf(__builtin_fmaf(-x, r, 1.0f), r, r);
+    return __builtin_amdgcn_classf(r, 0x198) ? refined : r;  // +-normal, +-denormal
+}
+__device__ __forceinline__ double reciprocal(double x) { return 1.0 / x; }
+
 __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackRecord &r) {
     const TriIds t = load_ids(a, j);
     const real *m = a.bary + 9 * (int64_t)t.tri;
@@ -60,8 +70,9 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
     for (int k = 0; k < 9; k++) r.m[k] = m[k];
     const real4 va = a.vertices[t.ia], vb = a.vertices[t.ib], vc = a.vertices[t.ic];
     r.w[0] = va.w; r.w[1] = vb.w; r.w[2] = vc.w;
-    r.iw[0] = 1.0f / va.w; r.iw[1] = 1.0f / vb.w; r.iw[2] = 1.0f / vc.w;
-    r.iw2[0] = 1.0f / (va.w * va.w); r.iw2[1] = 1.0f / (vb.w * vb.w); r.iw2[2] = 1.0f / (vc.w * vc.w);
+    // gradients only: 1 / w to within one unit in the last place, and its square for 1 / (w * w)
+    r.iw[0] = reciprocal(va.w); r.iw[1] = reciprocal(vb.w); r.iw[2] = reciprocal(vc.w);
+    r.iw2[0] = r.iw[0] * r.iw[0]; r.iw2[1] = r.iw[1] * r.iw[1]; r.iw2[2] = r.iw[2] * r.iw[2];
     r.op[0] = a.opacities[t.ia]; r.op[1] = a.opacities[t.ib]; r.op[2] = a.opacities[t.ic];
 #pragma unroll
     for (int k = 0; k < 3; k++) {
@@ -73,15 +84,6 @@ __device__ __forceinline__ void gather_back(const RasterArgs &a, int j, BackReco
     r.id[0] = t.ia; r.id[1] = t.ib; r.id[2] = t.ic;
 }
 
-// 1 / x to within one unit in the last place: the hardware estimate and one Newton step where
-// the estimate is an ordinary number (zero, infinity and NaN pass through as they are).  Used
-// where the reference divides in its backward pass and the quotient is no carried state.
-__device__ __forceinline__ float reciprocal(float x) {
-    const float r = __builtin_amdgcn_rcpf(x);
-    const float refined = __builtin_fmaf(__builtin_fmaf(-x, r, 1.0f), r, r);
-    return __builtin_amdgcn_classf(r, 0x198) ? refined : r;  // +-normal, +-denormal
-}
-__device__ __forceinline__ double reciprocal(double x) { return 1.0 / x; }
 
 // Reverse-traversal state of one pixel (render.cu:647-653).
 struct BackState {
@@ -231,6 +233,9 @@ __device__ __forceinline__ void fragment_terms(const FragSeed &f, const BackReco
         // reference's form: its differences of screen coordinates cancel, and for a sliver that rounding
         // is larger than the tolerance of the comparison, so the shorter closed form
         // (-l_v * row k of the matrix) does not reproduce the reference's numbers.
+        // Nor are they fused: a fused multiply-add moves l0..l2 by as much as the reference's own rounding
+        // does, which the numerators amplify for a sliver (measured: 11 rounding steps of the terms' magnitudes
+        // where 2 are allowed), and the same holds for v * denom - nom in interp_backward_scalar (2.6 steps).
         const real T = (bx - ax) * (cy - ay) - (by - ay) * (cx - ax);
         const real inv_T = reciprocal(T);
         const real l0 = ((bx - px) * (cy - py) - (by - py) * (cx - px)) * inv_T;
