@@ -367,58 +367,46 @@ __device__ __forceinline__ void wave_lds_sync() {
 
 // Adds up the runs of equal list entry among the first n slots of a wave's term matrix (row q = term
 // q, rows kTermStride apart; slots of one entry are neighbours) and adds every non-zero run sum to the
-// gradient arrays.  Bit c of `heads` is set where slot c starts a run.  First every lane (group, q)
-// turns its third of row q into running sums that start over at each head: no branch and no look at
-// the entries.  The last slot of a run, and of a third, then holds a sum to deliver; those slots are
-// taken three at a time, one per group.  vertex_at(c, v): vertex id v of the entry in slot c.
+// gradient arrays.  Bit c of `heads` is set where slot c starts a run.  Lane (group, q) owns a fixed third of
+// row q -- slots [0, 22), [22, 44) or [44, 64) -- and turns it into running sums that start over at each head:
+// straight-line code, no branch, no look at the entries; slots from n on hold what an earlier round left, which
+// a running sum carries to later slots only, never into a slot below n.  The last slot of a run, and of a third,
+// then holds a sum to deliver, and every lane walks the ones of its own third.  vertex_at(c, v): vertex id v of
+// the entry in slot c.
+constexpr int kRunSpan = 22;  // slots of a third (the last one has kWave - 2 * kRunSpan = 20)
 template <typename VertexAt>
 __device__ __forceinline__ void add_run_sums(real *terms, int n, uint64_t heads, const TermLane &t, VertexAt vertex_at) {
-    constexpr int kAhead = 8;  // terms read ahead, so that the LDS latency is paid once per eight slots
-    const int per = (n + 2) / 3;
-    const int c0 = min(t.group * per, n), c1 = min(c0 + per, n);
-    real *row = terms + t.q * kTermStride;
-    if (t.group < 3) {
-        const uint32_t mine = (uint32_t)(heads >> c0);  // per <= 22 slots
+    if (t.group >= 3) return;  // the one lane left over; nothing below synchronises the wave
+    const int c0 = t.group * kRunSpan;
+    real *row = terms + t.q * kTermStride + c0;
+    const bool full = t.group < 2;  // a third of kRunSpan slots
+    {
+        const uint32_t mine = (uint32_t)(heads >> c0);
+        real v[kRunSpan];
+#pragma unroll
+        for (int k = 0; k < kRunSpan; k++) v[k] = (k < kWave - 2 * kRunSpan || full) ? row[k] : 0.0f;
         real sum = 0.0f;
-        for (int i = 0; c0 + i < c1; i += kAhead) {
-            real v[kAhead];
 #pragma unroll
-            for (int k = 0; k < kAhead; k++) v[k] = row[min(c0 + i + k, c1 - 1)];
-#pragma unroll
-            for (int k = 0; k < kAhead; k++) {
-                if (c0 + i + k >= c1) break;
-                sum = ((mine >> (i + k)) & 1) ? v[k] : sum + v[k];
-                row[c0 + i + k] = sum;
-            }
+        for (int k = 0; k < kRunSpan; k++) {
+            sum = ((mine >> k) & 1) ? v[k] : sum + v[k];
+            if (k < kWave - 2 * kRunSpan || full) row[k] = sum;
         }
     }
-    wave_lds_sync();
-    uint64_t tails = (heads >> 1) | (1ull << (n - 1));
-    if (per < n) tails |= 1ull << (per - 1);
-    if (2 * per < n) tails |= 1ull << (2 * per - 1);
+    // what a lane reads below it wrote itself above: LDS serves a wave's instructions in order
+    uint64_t tails = (heads >> 1) | (1ull << (n - 1)) | (1ull << (kRunSpan - 1)) | (1ull << (2 * kRunSpan - 1));
     if (n < kWave) tails &= (1ull << n) - 1;
-    while (tails) {  // wave-uniform; six slots per turn, so that two chains of LDS reads are in flight per lane
-        int c[2] = {-1, -1};
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-#pragma unroll
-            for (int k = 0; k < 3; k++)
-                if (tails) {
-                    const int bit = __builtin_ctzll(tails);
-                    tails &= tails - 1;
-                    if (t.group == k) c[u] = bit;
-                }
-        real sum[2] = {0.0f, 0.0f};
-        int vertex[2] = {0, 0};
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-            if (c[u] >= 0) {
-                sum[u] = row[c[u]];
-                vertex[u] = vertex_at(c[u], t.vertex);
-            }
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-            if (sum[u] != 0.0f) unsafeAtomicAdd(t.base + (int64_t)t.stride * vertex[u], sum[u]);
+    uint32_t mine = (uint32_t)(tails >> c0) & ((1u << (full ? kRunSpan : kWave - 2 * kRunSpan)) - 1);
+    while (mine) {
+        // two slots per turn, so that two chains of LDS reads are in flight
+        const int k0 = __builtin_ctz(mine);
+        mine &= mine - 1;
+        const int k1 = mine ? __builtin_ctz(mine) : k0;
+        const bool two = mine != 0;
+        mine &= mine - 1;  // 0 & anything = 0
+        const real sum0 = row[k0], sum1 = two ? row[k1] : 0.0f;
+        const int vertex0 = vertex_at(c0 + k0, t.vertex), vertex1 = vertex_at(c0 + k1, t.vertex);
+        if (sum0 != 0.0f) unsafeAtomicAdd(t.base + (int64_t)t.stride * vertex0, sum0);
+        if (sum1 != 0.0f) unsafeAtomicAdd(t.base + (int64_t)t.stride * vertex1, sum1);
     }
 }
 
