@@ -446,16 +446,13 @@ __device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
 //      order inside an entry, so every (pixel, entry) hit of the wave owns one
 //      slot, slots are grouped by entry, and a lane's own hits have increasing
 //      numbers in the order it must visit them (reverse blend order);
-//   3. in rounds of 64 slots: lane = pixel hands its hits of the round to their slots;
-//      lane = slot evaluates the hit's own opacity, colour and view depth (no state in
-//      them, so every lane is busy); lane = pixel then walks its own slots in order
-//      and advances the pixel's transmittance and running sums, which turns the five
-//      values of a slot into the five numbers the gradient terms are linear in (only
-//      this short part runs as often as the busiest lane has hits in the round);
+//   3. ordered part, in rounds of 64 slots: every lane walks its own hits and
+//      advances the pixel's transmittance and running sums; each hit leaves
+//      five numbers in its slot;
 //   4. order-free part with every lane busy: lane = slot evaluates the 21 gradient
-//      terms of its hit (record and barycentrics still in registers from 3) and writes
-//      them to a term matrix; three groups of 21 lanes add up the runs of equal entry
-//      and issue one global floating-point atomic per run and term.
+//      terms of its hit and writes them to a term matrix; three groups of 21 lanes
+//      add up the runs of equal entry and issue one global floating-point atomic
+//      per run and term.
 template <int kLayout>
 __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(RasterArgs a, BackwardArgs g) {
     __shared__ BackRecord s_rec[kBackBatch];
@@ -582,8 +579,7 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
 
         for (uint32_t round0 = 0; round0 < n_hits; round0 += kWaveSlots) {
             const int n_slots = (int)min((uint32_t)kWaveSlots, n_hits - round0);
-            // 3a. lane = pixel: my hits of the round take their slots (increasing slot = the order I must visit them in)
-            uint64_t my_slots = 0;
+            // 3. ordered part, lane by lane over its own hits
             while (true) {
                 int e = -1;
                 uint32_t slot = 0;
@@ -600,68 +596,38 @@ __global__ __launch_bounds__(kTileThreads) void backward_tile_order_kernel(Raste
 #pragma unroll
                     for (int wd = 0; wd < kBackWords; wd++)
                         if ((e >> 6) == wd) m[wd] &= ~(1ull << (e & 63));
+                    const BackRecord &r = s_rec[e];
+                    real b0, b1, b2;
+                    bary_apply(r.m, p.px, p.py, b0, b1, b2);
+                    const FragSeed f = fragment_state_step(st, r, b0, b1, b2);
+                    // the five numbers wait in the slot's column of the term matrix, which is free until
+                    // the slot's own lane replaces them by the terms
+                    terms[0 * kTermStride + slot] = f.d_do;
+                    terms[1 * kTermStride + slot] = f.gc[0];
+                    terms[2 * kTermStride + slot] = f.gc[1];
+                    terms[3 * kTermStride + slot] = f.gc[2];
+                    terms[4 * kTermStride + slot] = f.dd_dz;
                     tags[slot] = e | (lane << 8);
-                    my_slots |= 1ull << slot;
-                }
-            }
-            wave_lds_sync();
-
-            // 3b. lane = slot: the fragment's own opacity, colour and view depth, with every lane busy; they wait
-            //     in the slot's column of the term matrix, which is free until the slot's lane writes its terms
-            const int packed = (lane < n_slots) ? tags[lane] : (lane << 8);
-            const int tag = (lane < n_slots) ? (packed & 0xff) : -1;
-            // the pixel of the slot, from the lane that owns it
-            const real px = __shfl(p.px, packed >> 8, kWave), py = __shfl(p.py, packed >> 8, kWave);
-            BackRecord r;
-            real b0 = 0.0f, b1 = 0.0f, b2 = 0.0f;
-            if (lane < n_slots) {
-                r = s_rec[tag];
-                bary_apply(r.m, px, py, b0, b1, b2);
-                const FragValue v = fragment_value(r, b0, b1, b2);
-                terms[0 * kTermStride + lane] = v.o;
-                terms[1 * kTermStride + lane] = v.color[0];
-                terms[2 * kTermStride + lane] = v.color[1];
-                terms[3 * kTermStride + lane] = v.color[2];
-                terms[4 * kTermStride + lane] = v.z;
-            }
-            wave_lds_sync();
-
-            // 3c. lane = pixel: the ordered part over my slots, which replaces the five values by the five
-            //     numbers the gradient terms are linear in
-            while (true) {
-                const bool active = my_slots != 0;
-                if (__builtin_amdgcn_ballot_w64(active) == 0) break;
-                if (active) {
-                    const int c = __builtin_ctzll(my_slots);
-                    my_slots &= my_slots - 1;
-                    FragValue v;
-                    v.o = terms[0 * kTermStride + c];
-                    v.color[0] = terms[1 * kTermStride + c];
-                    v.color[1] = terms[2 * kTermStride + c];
-                    v.color[2] = terms[3 * kTermStride + c];
-                    v.z = terms[4 * kTermStride + c];
-                    const FragSeed f = fragment_chain_step(st, v);
-                    terms[0 * kTermStride + c] = f.d_do;
-                    terms[1 * kTermStride + c] = f.gc[0];
-                    terms[2 * kTermStride + c] = f.gc[1];
-                    terms[3 * kTermStride + c] = f.gc[2];
-                    terms[4 * kTermStride + c] = f.dd_dz;
                 }
             }
             wave_lds_sync();
 
             // 4. order-free part: lane = slot
-            FragSeed f;
-            f.d_do = f.gc[0] = f.gc[1] = f.gc[2] = f.dd_dz = 0.0f;
+            int tag = -1;
+            if (lane < n_slots) tag = tags[lane] & 0xff;
+            // the pixel of the slot, from the lane that owns it
+            const int src = (lane < n_slots) ? tags[lane] >> 8 : lane;
+            const real px = __shfl(p.px, src, kWave), py = __shfl(p.py, src, kWave);
             if (lane < n_slots) {
+                FragSeed f;
                 f.d_do = terms[0 * kTermStride + lane];
                 f.gc[0] = terms[1 * kTermStride + lane];
                 f.gc[1] = terms[2 * kTermStride + lane];
                 f.gc[2] = terms[3 * kTermStride + lane];
                 f.dd_dz = terms[4 * kTermStride + lane];
-            }
-            wave_lds_sync();  // every slot's five numbers are in registers before terms take their place
-            if (lane < n_slots) {
+                const BackRecord &r = s_rec[tag];
+                real b0, b1, b2;
+                bary_apply(r.m, px, py, b0, b1, b2);
                 real term[kTerms];
                 fragment_terms(f, r, b0, b1, b2, px, py, term);
 #pragma unroll
