@@ -33,21 +33,22 @@ HBM_PEAK_GBS = 8000.0
 
 # Bytes per launch of sort_sweep_kernel that pass the L2 on their way to the fabric are measured with rocprofv3 --pmc (read
 # and write requests by size, and FETCH_SIZE / WRITE_SIZE scaled by a 256 MiB plain copy) and written into this summary as a
-# line "sort_sweep_kernel traffic_bytes_per_launch=<bytes> keys=<K> commit=<hash>"; the bench line quotes it only for that K.
+# lines "sort_sweep_kernel_traffic_bytes_per_launch=<bytes> keys=<K> commit=<hash>" and "lists_stage_traffic_bytes_per_frame=...";
+# the bench line quotes them only for that K.
 TRAFFIC_SUMMARY = os.path.join("profiles", "config2_hbm_traffic_counters.md")
 
 
-def measured_sweep_traffic(n_keys):
-    """-> (bytes per launch or None, where the figure comes from)"""
+def measured_traffic(what, n_keys):
+    """-> (bytes or None, where the figure comes from): the line `<what>=<bytes> keys=<K> commit=<hash>` of the summary"""
     try:
         text = open(os.path.join(ROOT, TRAFFIC_SUMMARY)).read()
     except OSError:
         return None, None
     for line in text.splitlines():
-        if line.startswith("sort_sweep_kernel traffic_bytes_per_launch="):
-            fields = dict(f.split("=", 1) for f in line.split()[1:])
+        if line.startswith(what + "="):
+            fields = dict(f.split("=", 1) for f in line.split())
             if int(fields.get("keys", -1)) == n_keys:
-                return float(fields["traffic_bytes_per_launch"]), f"{TRAFFIC_SUMMARY} @ {fields.get('commit', '?')}"
+                return float(fields[what]), f"{TRAFFIC_SUMMARY} @ {fields.get('commit', '?')}"
     return None, f"{TRAFFIC_SUMMARY} holds no measurement for K={n_keys}"
 
 
@@ -192,7 +193,8 @@ def main():
     # offsets read, 12 K written), the passes through memory, the per-tile depth sort (24 K), counts and offsets per tile
     moved_bytes = (60.0 + 52.0) * M + (52.0 * M + 12.0 * K) + 24.0 * passes_through_memory * K + 24.0 * K + 12.0 * (T + 1)
     sort_ms = sum(per_step.get(k, 0.0) for k in sort_kernels)
-    traffic, traffic_source = measured_sweep_traffic(K)
+    traffic, traffic_source = measured_traffic("sort_sweep_kernel_traffic_bytes_per_launch", K)
+    stage_traffic, stage_traffic_source = measured_traffic("lists_stage_traffic_bytes_per_frame", K)
 
     out = {
         "metric": "fwd+bwd frames/s (1M tris, 1920x1080)" if args.config == 2 else f"fwd+bwd frames/s (config {args.config})",
@@ -223,7 +225,8 @@ def main():
                                 "frac_of_hbm_peak": bin_sort_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
                                 "moved_bytes": moved_bytes,
                                 "moved_bytes_model": "what the kernels read and write by their access pattern (not counters)",
-                                "frac_of_hbm_peak_moved": moved_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS},
+                                "frac_of_hbm_peak_moved": moved_bytes / (bin_sort_ms / 1000.0) / 1e9 / HBM_PEAK_GBS,
+                                "traffic_bytes_by_counters": stage_traffic, "traffic_source": stage_traffic_source},
         "sort_in_frame": {"keys": K, "passes_through_memory": passes_through_memory, "passes_of_the_byte_model": model_passes,
                           "depth_bits": "sorted per tile in LDS: one more read and write of every pair",
                           "ms": sort_ms, "Gkeys_per_s": K / (sort_ms / 1000.0) / 1e9},
