@@ -307,6 +307,16 @@ def test_frame_route_with_more_than_65536_tiles(cuda, oracle):
     np.testing.assert_array_equal(u64(fkeys), want_keys)
     np.testing.assert_array_equal(fids.cpu().numpy(), want_vals)
     np.testing.assert_array_equal(foffsets.cpu().numpy(), oracle.tile_ranges(want_keys, T))
+    # the one-call binning with more than 256 tile columns: plain tile ids in the keys, the sort counts its own digits
+    assert _C.bin_frame_supported(d["vertices"], W, H, tw, th)
+    binned = _C.bin_frame(d["vertices"], d["indices"], W, H, tw, th)
+    assert int(binned["total_and_status"][0].item()) == K and int(binned["total_and_status"][1].item()) == 0
+    np.testing.assert_array_equal(np.sort(u64(binned["keys"][:K])), np.sort(em["keys64"]))
+    fkeys, fids, fstatus, foffsets = _C.build_frame_lists(binned, K)
+    assert int(fstatus.item()) == 0
+    np.testing.assert_array_equal(u64(fkeys), want_keys)
+    np.testing.assert_array_equal(fids.cpu().numpy(), want_vals)
+    np.testing.assert_array_equal(foffsets.cpu().numpy(), oracle.tile_ranges(want_keys, T))
 
 
 def test_one_frame_state_serves_two_sorting_calls(cuda):

@@ -329,7 +329,7 @@ def saved_blend_order(fragments, offsets, tile_width, tile_height):
 
 
 def bin_frame_supported(vertices, width, height, tile_width, tile_height):
-    """Whether tg_bin_frame takes this frame (float build, at most 65535 tile columns and rows, 2^21 tiles)."""
+    """Whether tg_bin_frame takes this frame (float build, at most 2^21 tiles)."""
     return _bits(vertices) == 32 and bool(_lib.load(32).tg_bin_frame_supported(width, height, tile_width, tile_height))
 
 
