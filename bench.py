@@ -308,10 +308,16 @@ def main():
         cores = min(O.max_threads(), len(os.sched_getaffinity(0)), 16)
         single, many = cpu_oracle_baseline(scene, MODES[args.mode], W, H, cores)
         out["cpu_baseline"] = {"value": 1.0 / many["forward_backward_seconds"], "unit": "frames/s", "cores": cores, "kind": "port",
+                               "mode": args.mode,
                                "sample": "the same frame, forward + backward: OpenMP over tiles after one warm-up, median of three "
                                          "runs (binning, sort and ranges are serial code); the single-thread figures are one run",
                                "openmp": many, "single_thread": dict(single, cores=1,
                                                                      value=1.0 / single["forward_backward_seconds"])}
+        # the other compositing mode on the same frame, same protocol
+        other = "A" if args.mode == "B" else "B"
+        single, many = cpu_oracle_baseline(scene, MODES[other], W, H, cores)
+        out["cpu_baseline"]["other_mode"] = {"mode": other, "value": 1.0 / many["forward_backward_seconds"], "cores": cores, "openmp": many,
+                                             "single_thread": dict(single, cores=1, value=1.0 / single["forward_backward_seconds"])}
     print(json.dumps(out))
 
 

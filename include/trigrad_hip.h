@@ -217,7 +217,13 @@ int tg_build_tile_lists(const tg_real *records, const uint32_t *tri_offsets, int
 /* tg_bin_frame = tg_bin_count + tg_scan_exclusive_u32 + tg_bin_emit in one call
  * and two launches (count_per_tile, the cumsum of per_tile_lists and
  * fill_per_tile_lists_kernel, render.cu:90-139, 202-270, 290-308): keys and
- * values as tg_bin_emit leaves them, total_and_status[0] = K.  The emission
+ * values in tg_bin_emit's order with tg_bin_emit's depth word,
+ * total_and_status[0] = K.  The high word of a key is the tile id only when the
+ * frame has more than 256 tile columns or rows; otherwise it is
+ * (tile row << column_bits) | tile column, column_bits = the bits that tell the
+ * frame's tile columns apart (7 for 120 columns): tg_build_frame_lists sorts by
+ * column, then by row, and its last pass writes the tile id, so the sorted keys
+ * are those of tg_sort_tile_lists either way.  The emission
  * reads K on the device, so the host does not have to know it in between: the
  * key buffers are the caller's guess, a key whose position is key_capacity or
  * more is not written, K is exact either way, and a caller who finds

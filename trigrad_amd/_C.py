@@ -310,7 +310,7 @@ def build_tile_lists(setup, n_keys, emit_only=False, prepared=None):
 
 # ---- the frame's route: binning in one launch -------------------------------------------------------------
 
-_frame_states = {}  # device index -> dict(frame, epoch): the state tg_bin_frame keeps between calls
+_frame_states = {}  # (device index, stream) -> dict(frame, epoch): the state tg_bin_frame keeps between calls
 _frame_lock = threading.Lock()
 _FRAME_TAIL = 256  # bytes behind the library's frame state: K and the status word of the binning
 
@@ -334,14 +334,16 @@ def bin_frame_supported(vertices, width, height, tile_width, tile_height):
 
 
 def _next_frame_state(dev, need):
-    """The device's frame state of at least `need` bytes, zeroed when it is made, and the epoch of the call about to
-    use it (they count up by one; a state whose epochs run out is replaced by a fresh one)."""
+    """The frame state of at least `need` bytes of the device's current stream, zeroed when it is made, and the epoch of
+    the call about to use it (they count up by one; a state whose epochs run out is replaced by a fresh one).  A state
+    per stream: frames on one stream follow each other, frames on two streams may run at the same time."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
     with _frame_lock:
-        st = _frame_states.get(dev.index)
+        st = _frame_states.get(key)
         if st is None or st["bytes"] < need or st["epoch"] >= 0x3FFFFFF0:
             size = need + need // 4
             st = dict(frame=torch.zeros((size + _FRAME_TAIL,), dtype=torch.uint8, device=dev), epoch=0, bytes=size)
-            _frame_states[dev.index] = st
+            _frame_states[key] = st
         st["epoch"] += 1
         return st["frame"], st["bytes"], st["epoch"]
 
