@@ -552,6 +552,45 @@ def test_ticketed_tile_numbers_change_nothing(cuda, oracle):
         assert torch.equal(a, b)
 
 
+def test_frames_on_two_streams_keep_their_own_state(cuda):
+    """Two streams render different frames at the same time (tickets on: the device is shared between them).  The
+    binning's state between calls -- epoch-stamped look-back words, alternating digit totals -- is kept per stream,
+    so every frame is what its stream gives alone."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import _C
+    import scenes as S
+    frames = []
+    for config in (1, 0):
+        scene = S.config(config)
+        d = to_device(scene, cuda)
+        frames.append((d, scene["width"], scene["height"]))
+
+    def render(k):
+        d, W, H = frames[k]
+        return trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, 16, 16, 1 / 256, False, False, -1)[0]
+
+    alone = [render(0), render(1)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=cuda), torch.cuda.Stream(device=cuda)]
+    got = [[], []]
+    try:
+        _C.force_tickets(True)
+        for _ in range(6):
+            for k in (0, 1):
+                with torch.cuda.stream(streams[k]):
+                    got[k].append(render(k))
+        torch.cuda.synchronize()
+        trigrad_amd.verify_frames()
+    finally:
+        _C.force_tickets(False)
+    states = {key for key in _C._frame_states if key[0] == cuda.index}
+    assert len({key[1] for key in states}) >= 3  # the default stream's and the two streams' own
+    for k in (0, 1):
+        for image in got[k]:
+            assert torch.equal(image, alone[k])
+
+
 @pytest.mark.parametrize("mode", ["A_default", "B_unlimited"])
 def test_scene_without_a_single_key(mode, cuda):
     """M >= 1 but K = 0 (every triangle degenerate): transparent image, infinite depth, zero gradients."""
