@@ -338,3 +338,33 @@ def test_one_frame_state_serves_two_sorting_calls(cuda):
         assert torch.equal(a, b)
     skeys = u64(first[0])
     assert (np.diff(skeys.astype(np.uint64).view(np.int64)) >= 0).all()
+
+
+def test_key_buffers_smaller_than_the_frame_needs(cuda, oracle):
+    """tg_bin_frame with a key capacity below K: K comes back exact, the keys that fit are the first ones of the emission
+    order, nothing is written behind the capacity; and a frame whose guess of K was too small is binned again."""
+    import torch
+    import trigrad_amd
+    from trigrad_amd import _C
+    import scenes as S
+    scene = S.random_soup(900, 200, 150, seed=21, sigma_px=9.0, varying_w=True)
+    W, H, tw, th = 200, 150, 16, 16
+    d = to_device(scene, cuda)
+    em = oracle.bin_emit(scene["vertices"], scene["indices"], W, H, tw, th)
+    K = em["keys64"].shape[0]
+    full = _C.bin_frame(d["vertices"], d["indices"], W, H, tw, th, capacity=K + 100)
+    assert int(full["total_and_status"][0].item()) == K
+    capacity = K // 3
+    small = _C.bin_frame(d["vertices"], d["indices"], W, H, tw, th, capacity=capacity)
+    assert small["keys"].numel() == capacity
+    assert int(small["total_and_status"][0].item()) == K and int(small["total_and_status"][1].item()) == 0
+    assert torch.equal(small["keys"], full["keys"][:capacity]) and torch.equal(small["values"], full["values"][:capacity])
+    np.testing.assert_array_equal(full["values"][:K].cpu().numpy(), em["tri"])
+    with pytest.raises(ValueError):
+        _C.build_frame_lists(small, K)
+    # the whole frame with a guess of K that is far too small: the same image as with a good one
+    good = trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, 1 / 256, False, False, -1)[0]
+    _C._key_count_hint[cuda.index] = 7
+    again = trigrad_amd.render(d["vertices"], d["indices"], d["colors"], d["opacities"], W, H, tw, th, 1 / 256, False, False, -1)[0]
+    assert torch.equal(good, again)
+    assert _C._key_count_hint[cuda.index] == K
