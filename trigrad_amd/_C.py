@@ -36,8 +36,13 @@ def _ptr(t):
     return None if t is None else C.c_void_p(t.data_ptr())
 
 
+def _raw_stream(dev):
+    """The hipStream_t of the device's current torch stream, as an int (no Stream object is made)."""
+    return torch._C._cuda_getCurrentRawStream(dev.index)
+
+
 def _stream(t):
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    return C.c_void_p(_raw_stream(t.device))
 
 
 class _on_device:
@@ -337,7 +342,7 @@ def _next_frame_state(dev, need):
     """The frame state of at least `need` bytes of the device's current stream, zeroed when it is made, and the epoch of
     the call about to use it (they count up by one; a state whose epochs run out is replaced by a fresh one).  A state
     per stream: frames on one stream follow each other, frames on two streams may run at the same time."""
-    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    key = (dev.index, _raw_stream(dev))
     with _frame_lock:
         st = _frame_states.get(key)
         if st is None or st["bytes"] < need or st["epoch"] >= 0x3FFFFFF0:
