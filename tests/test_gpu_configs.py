@@ -6,8 +6,8 @@ bit-exact; image within 1e-5 absolute (and, since the forward arithmetic is the
 oracle's operation for operation, bit-identical); gradients of the L2 loss
 against the seeded target within 1e-4 relative + 1e-6 absolute, both for the
 loss as the benchmark defines it (mean) and, so that the absolute term does not
-make the check vacuous, for the summed loss with the absolute term scaled to
-the gradient's magnitude.
+make the check vacuous, for the summed loss, where two float32 rounding steps of
+the magnitudes of the element's own terms (from the oracle) are allowed on top.
 
 Size-independent properties checked on the GPU results alone: keys sorted,
 ranges monotone with offsets[T] = K = sum of counts, payload multiset = emitted
@@ -70,7 +70,18 @@ def test_binning_sort_ranges_full_size(cfg, cuda, oracle):
     ref_offsets, ref_ids, _ = oracle.per_tile_lists(v, idx, W, H)
     np.testing.assert_array_equal(offsets, ref_offsets)
     np.testing.assert_array_equal(sv, ref_ids)
-    # the route the frame takes (one pass for count + scan, emission from records, tile-list sort)
+    # the route the frame takes: count + scan, then the emission without a host wait; tile passes by column and row
+    binned = _C.bin_frame(d["vertices"], d["indices"], W, H, 16, 16, capacity=K + 1000)
+    assert binned["total_and_status"].tolist() == [K, 0]
+    np.testing.assert_array_equal(binned["values"][:K].cpu().numpy(), em["tri"])
+    np.testing.assert_array_equal(u64(binned["keys"][:K]) & np.uint64(0xFFFFFFFF), em["keys64"] & np.uint64(0xFFFFFFFF))  # depth words
+    fkeys, fids, fstatus, foffsets = _C.build_frame_lists(binned, K)
+    assert int(fstatus.item()) == 0
+    np.testing.assert_array_equal(u64(fkeys), sk)
+    np.testing.assert_array_equal(fids.cpu().numpy(), sv)
+    np.testing.assert_array_equal(foffsets.cpu().numpy(), ref_offsets)
+    del binned, fkeys, fids, foffsets
+    # the two-call route (count + scan in one pass, the host reads K, emission from records, tile-list sort)
     setup = _C.bin_setup(d["vertices"], d["indices"], W, H, 16, 16)
     assert setup["total_and_status"].tolist() == [K, 0]
     np.testing.assert_array_equal(setup["tri_offsets"].cpu().numpy(), offs.cpu().numpy())
@@ -175,4 +186,5 @@ def test_stage_timings_describe_the_frame_that_runs(cuda):
             sums.append(sum(timings.values()))
         a, b = float(np.median(untimed)), float(np.median(sums))
         kinds[pps] = (a, b)
+        print(f"per_pixel_sort={pps}: untimed forward {a * 1e3:.3f} ms, stages add up to {b * 1e3:.3f} ms")
         assert abs(b - a) <= 0.1 * a, f"per_pixel_sort={pps}: stages add up to {b * 1e3:.3f} ms, an untimed forward pass takes {a * 1e3:.3f} ms"
