@@ -428,6 +428,12 @@ __device__ __forceinline__ uint64_t transpose_bits(uint64_t x, int lane) {
     return x;
 }
 
+__device__ __forceinline__ int wave_max_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
 __device__ __forceinline__ uint32_t lanes_below_mask(uint64_t mask) {
     return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
@@ -815,10 +821,8 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     const PixelCoord p = pixel_of_thread(a, tile_id);
     const int rel_bits = 32 - __builtin_clz(max(end - start - 1, 1));  // bits that tell two list positions apart
     real *terms = s_term[wave];
-    int *rels = s_rel[wave];
     int *tags = s_tag[wave];
     int *vertices = s_vertex[wave];
-    uint8_t *srcs = s_src[wave];
     const TermLane tl = term_lane<kLayout>(g, lane);
 
     BackState st;
@@ -829,37 +833,74 @@ __global__ __launch_bounds__(kTileThreads) void backward_saved_order_kernel(Rast
     }
     const int64_t plane = (int64_t)a.W * a.H;
     const bool long_list = end - start > 0xffff;  // then the positions' high halves were saved as well
-    auto position_of_step = [&](int s) {
-        if (s >= n) return 0;
-        const int64_t at = (int64_t)(n - 1 - s) * plane + p.index;
-        const int low = g.fragments[at];
-        return long_list ? low | ((int)g.fragments[(int64_t)a.max_layers * plane + at] << 16) : low;
+    // The list positions of my steps, one after the other: step s is layer n - 1 - s, a plane further down each time.
+    const uint16_t *next_layer = g.fragments + ((int64_t)(n - 1) * plane + (p.valid ? p.index : 0));
+    const int64_t high_halves = (int64_t)a.max_layers * plane;
+    int steps_read = 0;
+    auto next_position = [&]() {
+        int position = -1;  // no such step: below every threshold
+        if (steps_read < n) {
+            position = *next_layer;
+            if (long_list) position |= (int)next_layer[high_halves] << 16;
+        }
+        next_layer -= plane;
+        steps_read++;
+        return position;
     };
     // the list positions of my next four steps
-    int ahead0 = position_of_step(0), ahead1 = position_of_step(1), ahead2 = position_of_step(2), ahead3 = position_of_step(3);
-    const int total = __builtin_amdgcn_readlane((int)wave_inclusive_scan_u32((uint32_t)n), kWave - 1);
+    int ahead0 = next_position(), ahead1 = next_position(), ahead2 = next_position(), ahead3 = next_position();
+    int remaining = __builtin_amdgcn_readlane((int)wave_inclusive_scan_u32((uint32_t)n), kWave - 1);  // the wave's fragments not handed out yet
 
-    int step = 0, step_base = 0;  // wave-uniform: the first step with a slot left, and the number of its first slot
-    for (int round0 = 0; round0 < total; round0 += kWave) {
-        const int n_slots = min(kWave, total - round0);
-        // 1. the round's slots
-        uint64_t mine = 0;  // my slots of the round: increasing slot = increasing step
-        while (step_base < round0 + kWave) {
-            const uint64_t votes = __builtin_amdgcn_ballot_w64(n > step);
-            if (votes == 0) break;
-            const int count = __builtin_popcountll(votes);
-            const int slot = step_base + (int)lanes_below_mask(votes) - round0;
-            if (n > step && slot >= 0 && slot < kWave) {
-                mine |= 1ull << slot;
-                rels[slot] = ahead0;
-                srcs[slot] = (uint8_t)lane;
-                ahead0 = ahead1; ahead1 = ahead2; ahead2 = ahead3;
-                ahead3 = position_of_step(step + 4);
+    // How many of my next steps lie at or above list position `threshold`: a prefix of them, so that I visit them in order.
+    // -> the four masks of the lanes whose first, second, ... next step qualifies, and the slots that makes.
+    auto slots_at = [&](int threshold) {
+        const uint64_t first = __builtin_amdgcn_ballot_w64(ahead0 >= threshold);
+        const uint64_t second = first & __builtin_amdgcn_ballot_w64(ahead1 >= threshold);
+        const uint64_t third = second & __builtin_amdgcn_ballot_w64(ahead2 >= threshold);
+        const uint64_t fourth = third & __builtin_amdgcn_ballot_w64(ahead3 >= threshold);
+        return __builtin_popcountll(first) + __builtin_popcountll(second) + __builtin_popcountll(third) + __builtin_popcountll(fourth);
+    };
+
+    for (int round = 0; remaining > 0; round++) {
+        // 1. the round's slots.  A round takes the wave's pending fragments from the far end of the tile's LIST, not step s
+        //    of every pixel: a triangle is at another step in each pixel it covers, but at one list position, so the
+        //    slots of a round then hold few different entries -- long runs, few atomics, and gathers whose lanes share
+        //    their cache lines.  Every pixel gives a prefix of its next (at most four) steps, those at or above a
+        //    threshold: the largest threshold that fills the 64 slots.  What overflows is cut off in lane order from a
+        //    start lane that moves from round to round, and waits for the next round.
+        int threshold = 0, offered = slots_at(0);
+        if (offered > kWave) {
+            int high = __builtin_amdgcn_readfirstlane(wave_max_i32(ahead0)) + 1;  // slots_at(threshold) >= 64 > slots_at(high) = 0
+            while (high - threshold > 1) {
+                const int middle = threshold + (high - threshold) / 2;
+                const int slots = slots_at(middle);
+                if (slots >= kWave) { threshold = middle; offered = slots; } else { high = middle; }
             }
-            if (step_base + count > round0 + kWave) break;  // the step goes on in the next round
-            step_base += count;
-            step++;
         }
+        const bool first = ahead0 >= threshold, second = first && ahead1 >= threshold, third = second && ahead2 >= threshold,
+                   fourth = third && ahead3 >= threshold;
+        const int mine_count = (int)first + (int)second + (int)third + (int)fourth;
+        const int taken_incl = (int)wave_inclusive_scan_u32((uint32_t)mine_count);
+        const int first_lane = (round * 23) & (kWave - 1);
+        const int before_first = __builtin_amdgcn_readlane(taken_incl - mine_count, first_lane);
+        int base = taken_incl - mine_count - before_first;
+        if (lane < first_lane) base += offered;
+        const int granted = max(0, min(mine_count, kWave - base));
+        const int n_slots = min(kWave, offered);
+        int *rels = s_rel[wave];
+        uint8_t *srcs = s_src[wave];
+        if (granted > 0) { rels[base] = ahead0; srcs[base] = (uint8_t)lane; }
+        if (granted > 1) { rels[base + 1] = ahead1; srcs[base + 1] = (uint8_t)lane; }
+        if (granted > 2) { rels[base + 2] = ahead2; srcs[base + 2] = (uint8_t)lane; }
+        if (granted > 3) { rels[base + 3] = ahead3; srcs[base + 3] = (uint8_t)lane; }
+        uint64_t mine = granted > 0 ? ((1ull << granted) - 1) << base : 0ull;  // my slots of the round: increasing slot = increasing step
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (granted > k) {
+                ahead0 = ahead1; ahead1 = ahead2; ahead2 = ahead3;
+                ahead3 = next_position();
+            }
+        remaining -= n_slots;
         wave_lds_sync();
 
         // 2. lane = slot: the record, and the fragment's own values
