@@ -786,13 +786,14 @@ __global__ __launch_bounds__(kTileThreads) void backward_pixel_order_kernel(Rast
 // Per-pixel order with the blend order saved by the forward pass
 // (max_layers <= TG_MAX_SAVED_LAYERS): no re-selection.  Step s of a pixel is its
 // fragment n - 1 - s, so every pixel starts at its own far end.  The pixels of a wave
-// hold different numbers of fragments, so the (pixel, step) pairs of the wave are
-// numbered step by step, the pixels that still have a fragment in lane order inside a
-// step, and taken 64 at a time: a round's 64 slots keep every lane busy whatever
-// the pixels' counts are, and a pixel's own slots come in the order it must visit
-// them.  Per round:
-//   1. lane = pixel: which of my steps own a slot of the round; their list positions
-//      (fetched from the saved order a few steps ahead) go to the slots;
+// hold different numbers of fragments, so the wave takes its (pixel, step) pairs 64 at a
+// time: a round's 64 slots keep every lane busy whatever the pixels' counts are.  A round
+// takes the pending pairs nearest the far end of the tile's list (every pixel a prefix of
+// its next steps, so its own slots come in the order it must visit them): the slots of a
+// round then hold few different entries.  Per round:
+//   1. lane = pixel: which of my next steps (their list positions are fetched from the
+//      saved order four steps ahead) lie at or above the round's threshold; they get
+//      consecutive slots;
 //   2. lane = slot: gathers the record of its fragment from memory (neighbouring
 //      pixels hold the same few entries, so the loads hit in cache; staging the tile's
 //      records in LDS first was measured slower, for the workgroups per CU it costs)
